@@ -1,0 +1,150 @@
+/*
+ * trinity_hip.h -- C ABI of libtrinity_hip.so: hand-written gfx950 (MI355X) kernels for the
+ * fused operators that the reference's code generator emits at run time.
+ *
+ * Boundary being replaced.  In the reference a generated Python module exposes
+ * `forward(*tensors, **block_sizes)` (TritonGen.py:568-712) whose body launches
+ * `kernel_i[grid](ptr, ptr.stride(0), ..., M=..., N=..., D=..., H=..., P=...)` on the
+ * caller's current stream (TritonGen.py:590-708).  Each function below is what one such
+ * launch becomes: plain device pointers, element strides and sizes in; results written in
+ * place into caller-owned buffers; enqueued on the stream handle given; nothing allocated,
+ * nothing synchronised, no host read of device memory -- so a call may sit inside a HIP
+ * graph capture exactly as the reference's callers capture `forward`
+ * (vanilla_llama_benchmark.py:254-285).
+ *
+ * Conventions
+ *   - All tensors are fp16 unless a parameter says float.  Innermost (feature) stride is 1.
+ *   - Strides are in ELEMENTS.  Base pointers and row pitches must be 16-byte aligned
+ *     (128-bit loads); otherwise TRN_E_ALIGN.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).
+ *   - Every function returns TRN_OK or a negative trn_status; it never throws or aborts.
+ *   - Query head h reads KV head h / (n_q_heads / n_kv_heads)  (GQA / MQA).
+ *   - Causal with seq_q < seq_kv: query i sees keys j <= i + (seq_kv - seq_q)  (cached prefix).
+ */
+#ifndef TRINITY_HIP_H
+#define TRINITY_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum trn_status {
+    TRN_OK            =  0,
+    TRN_E_NULL        = -1,  /* a required pointer is NULL                              */
+    TRN_E_SHAPE       = -2,  /* a size is <= 0, not a supported multiple, or inconsistent */
+    TRN_E_STRIDE      = -3,  /* a stride is too small for the shape                       */
+    TRN_E_ALIGN       = -4,  /* pointer or pitch not 16-byte aligned                      */
+    TRN_E_UNSUPPORTED = -5,  /* e.g. head_dim not in {64,128}                             */
+    TRN_E_LAUNCH      = -6,  /* the HIP runtime refused the launch                        */
+    TRN_E_ARCH        = -7   /* current device is not gfx950                              */
+} trn_status;
+
+/* Library version (major*10000 + minor*100 + patch). */
+int trn_version(void);
+
+/* Static string naming a trn_status value ("TRN_E_SHAPE"...). */
+const char* trn_status_name(int status);
+
+/* 0 if the current HIP device is a gfx950, TRN_E_ARCH otherwise.  Not capture-safe
+ * (queries device properties); call once at load time. */
+int trn_check_device(void);
+
+/*
+ * RMSNorm rows:  y[r,:] = x[r,:] * rsqrt(mean(x[r,:]^2) + eps) * gamma[:]
+ * Replaces the arithmetic of ref_attn.py:348-350 (eps + weight form) and ref_rms.py:102-103
+ * (gamma == NULL, eps == 0).  fp32 mean-square; x is read once and y written once.
+ *
+ * Rows are addressed in two levels so the same kernel serves per-head normalisation of a
+ * [heads, seq, head_dim] tensor from row `row_start` on (ref_rms.py:217-222: only the
+ * newly appended keys are normalised):
+ *     row r -> outer = r / inner_rows, inner = r % inner_rows
+ *     x + outer*x_outer_stride + (row_start + inner)*ldx ;  y likewise.
+ * A plain [rows, cols] matrix is outer_rows = 1, inner_rows = rows, row_start = 0.
+ * cols must be a multiple of 8 and <= 16384.
+ */
+int trn_rmsnorm_f16(const void* x, const void* gamma /* nullable */, void* y,
+                    int64_t outer_rows, int64_t inner_rows, int64_t cols,
+                    int64_t x_outer_stride, int64_t ldx,
+                    int64_t y_outer_stride, int64_t ldy,
+                    int64_t row_start, float eps, void* stream);
+
+/* Shape / layout of one attention problem.  q,o: [batch, n_q_heads, seq_q, head_dim];
+ * k,v: [batch, n_kv_heads, seq_kv, head_dim]; any of them may be a strided view
+ * (e.g. token-major [batch, seq, heads*head_dim] has *_stride_h = head_dim). */
+typedef struct trn_attn_desc {
+    int32_t batch, n_q_heads, n_kv_heads, seq_q, seq_kv, head_dim;
+    int64_t q_stride_b, q_stride_h, q_stride_s;
+    int64_t k_stride_b, k_stride_h, k_stride_s;
+    int64_t v_stride_b, v_stride_h, v_stride_s;
+    int64_t o_stride_b, o_stride_h, o_stride_s;
+    float   scale;        /* multiplies Q K^T; the reference classes use 1 (ref_rms.py:77) */
+    int32_t causal;       /* 0: every query sees every key (ref_rms.py:78); 1: causal      */
+    /* Fused per-head RMSNorm of Q over head_dim before Q K^T (ref_rms.py:217-219). */
+    int32_t q_norm;       /* 0 off, 1 on                                                   */
+    float   q_norm_eps;
+    /* KeyFormer perturbation (ref_rms.py:172): z = (scale*QK^T + noise) / tau.            */
+    int64_t noise_stride_b, noise_stride_h, noise_stride_s;   /* noise [b, hq, seq_q, seq_kv] float */
+    float   tau;
+} trn_attn_desc;
+
+/*
+ * O = softmax(scale * Q K^T [+ causal mask]) V, fp32 softmax and accumulation, one pass over
+ * K/V with online softmax (no S x S intermediate).  Replaces the kernels generated for
+ * ref_rms.py:77-80 (Vanila), :225-228 (QKNorm, with q_norm=1 and K normalised beforehand by
+ * trn_rmsnorm_f16), and the attention half of :121-124 (PreNorm), :171-176 (KeyFormer),
+ * :272-277 (RoCo).
+ *
+ *   lse        nullable float [batch, n_q_heads, seq_q] (contiguous): natural-log row
+ *              normaliser log sum_j exp(s_ij), needed by trn_attn_colstats_f16.
+ *   gamma_q    nullable fp16 [head_dim]: weight of the fused Q norm (used when q_norm=1).
+ *   noise      nullable float: when given, the kernel also reduces the row normaliser of the
+ *              perturbed scores z into lse_pert (same shape as lse; required then).
+ */
+int trn_attn_fwd_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                     void* o, float* lse, const void* gamma_q,
+                     const float* noise, float* lse_pert, void* stream);
+
+/*
+ * Per-key column statistics of the attention probabilities, given the row normalisers from
+ * trn_attn_fwd_f16:   p_ij = exp(t_ij - lse_i),  out_sum[j] = sum_i p_ij,
+ * out_sumsq[j] = sum_i p_ij^2, over the queries i that can see key j.
+ *   noise == NULL : t = scale*QK^T, lse = plain row LSE           (RoCo, ref_rms.py:274-275)
+ *   noise != NULL : t = (scale*QK^T + noise)/tau, lse = lse_pert  (KeyFormer, ref_rms.py:172-174,
+ *                   summed over queries as the generated kernel's C_out is,
+ *                   keyformer_llama_benchmark.py:79)
+ * out_sum, out_sumsq (nullable): float [batch, n_q_heads, seq_kv] contiguous.  Deterministic
+ * (one workgroup owns a column block; no atomics).  v/o strides of desc are ignored.
+ */
+int trn_attn_colstats_f16(const trn_attn_desc* desc, const void* q, const void* k,
+                          const float* lse, const void* gamma_q, const float* noise,
+                          float* out_sum, float* out_sumsq, void* stream);
+
+/*
+ * Fused RMSNorm + Q/K/V projection:  Xn = RMSNorm(X; gamma, eps);  Q = Xn Wq, K = Xn Wk,
+ * V = Xn Wv  (X @ W, W is [hidden, n_out] row-major -- ref_rms.py:105-107, and the per-head
+ * column slices of convert_eval_rms.py:132-138).  The row mean-square is reduced inside the
+ * GEMM from the X tiles it streams, and applied as a row scale on the fp32 accumulator.
+ * norm == 0 skips the normalisation (ref_rms.py:47-49).
+ *
+ * Each output is written "head-split": element (token t, column n) of projection P goes to
+ *     P + (n / head_dim) * p_stride_h + t * p_stride_s + (n % head_dim)
+ * so the same call can write token-major [T, H*D] (stride_h = head_dim, stride_s = H*D),
+ * head-major [H, T, D], or rows P.. of a [H, P+M, D] KV cache (ref_rms.py:72-73).
+ * hidden, n_q, n_kv multiples of 8; head_dim a multiple of 8.
+ */
+int trn_prenorm_qkv_f16(const void* x, const void* gamma /* nullable */,
+                        const void* wq, const void* wk, const void* wv,
+                        void* q, void* k, void* v,
+                        int64_t tokens, int64_t hidden, int64_t n_q, int64_t n_kv, int64_t head_dim,
+                        int64_t ldx, int64_t ldwq, int64_t ldwk, int64_t ldwv,
+                        int64_t q_stride_h, int64_t q_stride_s,
+                        int64_t k_stride_h, int64_t k_stride_s,
+                        int64_t v_stride_h, int64_t v_stride_s,
+                        float eps, int32_t norm, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRINITY_HIP_H */

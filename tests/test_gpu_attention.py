@@ -1,0 +1,139 @@
+"""GPU parity: trn_attn_fwd_f16 (through the C ABI) against the CPU oracle.
+Tolerance for fp16 attention outputs: atol 2e-2, rtol 1e-2; LSE fp32: 1e-3 relative + 1e-3 abs."""
+import pytest
+import torch
+
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+ATOL, RTOL = 2e-2, 1e-2
+
+
+def close(got, want, atol=ATOL, rtol=RTOL):
+    got = got.float().cpu(); want = want.float()
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bad.any(), f"{int(bad.sum())} elements off; max abs err {err.max():.4g}"
+    return err.max().item()
+
+
+def make(B, Hq, Hkv, Sq, Skv, D, seed=42, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    q = ref.randn_half((B, Hq, Sq, D), g, 0, std)
+    k = ref.randn_half((B, Hkv, Skv, D), g, 0, std)
+    v = ref.randn_half((B, Hkv, Skv, D), g, 0, std)
+    return q, k, v
+
+
+CASES = [
+    # B, Hq, Hkv, Sq, Skv, D, causal
+    (1, 4, 2, 128, 128, 128, True),
+    (1, 4, 2, 128, 128, 128, False),
+    (2, 8, 2, 512, 512, 128, True),
+    (1, 2, 1, 300, 300, 128, True),      # ragged
+    (1, 3, 1, 77, 77, 64, True),         # MQA, D=64, ragged
+    (1, 6, 1, 256, 256, 64, True),
+    (1, 4, 4, 16, 1040, 128, False),     # the reference's decode-append shape (M=16, P=1024)
+    (1, 4, 4, 16, 1040, 128, True),      # causal with a cached prefix
+    (1, 5, 5, 16, 1040, 64, False),
+    (1, 2, 2, 1, 1, 64, True),
+    (1, 2, 1, 129, 257, 128, True),
+]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", CASES)
+def test_attention_parity(B, Hq, Hkv, Sq, Skv, D, causal):
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D)
+    scale = D ** -0.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    od = torch.zeros_like(qd)
+    lse = torch.zeros(B, Hq, Sq, dtype=torch.float32, device="cuda")
+    ops.attention(qd, kd, vd, od, scale, causal, lse=lse)
+    torch.cuda.synchronize()
+    want, want_lse = ref.attention(q, k, v, scale, causal, return_lse=True)
+    close(od, want)
+    close(lse, want_lse, atol=1e-3, rtol=1e-3)
+
+
+def test_attention_reference_recipe_unscaled():
+    """The reference's own input recipe and semantics: scale 1, no mask (ref_rms.py:77-78)."""
+    from triton_amd import ops
+    g = torch.Generator().manual_seed(42)
+    q = ref.reference_recipe((1, 8, 16, 128), g); k = ref.reference_recipe((1, 8, 1040, 128), g)
+    v = ref.reference_recipe((1, 8, 1040, 128), g)
+    od = torch.zeros_like(q).cuda()
+    ops.attention(q.cuda(), k.cuda(), v.cuda(), od, 1.0, False)
+    torch.cuda.synchronize()
+    close(od, ref.attention(q, k, v, 1.0, False), atol=1e-4, rtol=1e-2)
+
+
+def test_attention_closed_forms_on_gpu():
+    from triton_amd import ops
+    q, k, v = make(1, 4, 2, 200, 200, 128, seed=7)
+    od = torch.zeros_like(q).cuda()
+    ops.attention(torch.zeros_like(q).cuda(), k.cuda(), v.cuda(), od, 0.1, True)
+    torch.cuda.synchronize()
+    want = (v.float().repeat_interleave(2, 1).cumsum(2) / torch.arange(1, 201).view(1, 1, 200, 1))
+    close(od, want, atol=2e-3, rtol=2e-3)            # Q = 0: running mean of V
+    ops.attention(q.cuda(), k.cuda(), v.cuda(), od, 0.1, True)
+    torch.cuda.synchronize()
+    assert torch.equal(od[:, :, 0].cpu(), v.repeat_interleave(2, 1)[:, :, 0])   # row 0 sees only key 0
+
+
+def test_attention_token_major_views():
+    """q/o as views of token-major [B,S,H*D] buffers (the PreNorm block's layout)."""
+    from triton_amd import ops
+    B, Hq, Hkv, S, D = 1, 4, 2, 192, 128
+    q, k, v = make(B, Hq, Hkv, S, S, D, seed=3)
+    qt = q.permute(0, 2, 1, 3).contiguous().cuda()       # [B,S,H,D]
+    kt = k.permute(0, 2, 1, 3).contiguous().cuda(); vt = v.permute(0, 2, 1, 3).contiguous().cuda()
+    ot = torch.zeros_like(qt)
+    ops.attention(qt.permute(0, 2, 1, 3), kt.permute(0, 2, 1, 3), vt.permute(0, 2, 1, 3), ot.permute(0, 2, 1, 3),
+                  D ** -0.5, True)
+    torch.cuda.synchronize()
+    close(ot.permute(0, 2, 1, 3), ref.attention(q, k, v, D ** -0.5, True))
+
+
+def test_qnorm_fused():
+    from triton_amd import ops
+    B, Hq, Hkv, S, D = 1, 5, 1, 160, 64
+    q, k, v = make(B, Hq, Hkv, S, S, D, seed=11)
+    g = torch.Generator().manual_seed(5)
+    gq = ref.randn_half((D,), g, 1.0, 0.02); gk = ref.randn_half((D,), g, 1.0, 0.02)
+    kd = k.cuda(); kn = torch.empty_like(kd)
+    ops.head_rmsnorm(kd.view(B * Hkv, S, D), gk.cuda(), kn.view(B * Hkv, S, D), 1e-5)
+    od = torch.zeros_like(q).cuda()
+    ops.attention(q.cuda(), kn, v.cuda(), od, D ** -0.5, True, q_norm=True, gamma_q=gq.cuda(), q_eps=1e-5)
+    torch.cuda.synchronize()
+    close(od, ref.qknorm_attention(q, k, v, gq, gk, 1e-5, D ** -0.5, True))
+
+
+def test_noise_row_normaliser():
+    from triton_amd import ops
+    B, Hq, Hkv, S, D = 1, 4, 2, 200, 128
+    q, k, v = make(B, Hq, Hkv, S, S, D, seed=13)
+    noise = ref.gumbel_noise((B, Hq, S, S), 1234)
+    od = torch.zeros_like(q).cuda()
+    lse = torch.zeros(B, Hq, S, device="cuda"); lsep = torch.zeros(B, Hq, S, device="cuda")
+    tau, scale = 1.5, D ** -0.5
+    ops.attention(q.cuda(), k.cuda(), v.cuda(), od, scale, True, lse=lse, noise=noise.cuda(), tau=tau, lse_pert=lsep)
+    torch.cuda.synchronize()
+    close(od, ref.attention(q, k, v, scale, True))
+    s = ref.scores_fp32(q, k, scale, True)
+    close(lsep, torch.logsumexp((s + noise) / tau, -1), atol=1e-3, rtol=1e-3)
+    close(lse, torch.logsumexp(s, -1), atol=1e-3, rtol=1e-3)
+
+
+def test_attention_bad_arguments():
+    from triton_amd import ops, _lib
+    q, k, v = make(1, 2, 2, 8, 8, 32)
+    with pytest.raises(_lib.TrnError) as e:
+        ops.attention(q.cuda(), k.cuda(), v.cuda(), torch.zeros_like(q).cuda(), 1.0, False)
+    assert e.value.status_name == "TRN_E_UNSUPPORTED"
+    q, k, v = make(1, 3, 2, 8, 8, 64)
+    with pytest.raises(_lib.TrnError):
+        ops.attention(q.cuda(), k.cuda(), v.cuda(), torch.zeros_like(q).cuda(), 1.0, False)
+    q, k, v = make(1, 2, 2, 8, 4, 64)
+    with pytest.raises(_lib.TrnError):
+        ops.attention(q.cuda(), k.cuda(), v.cuda(), torch.zeros_like(q).cuda(), 1.0, True)   # causal, Skv < Sq

@@ -1,0 +1,59 @@
+// Shared device helpers for the gfx950 kernels: vector types, MFMA wrappers, wave utilities.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "../../include/trinity_hip.h"
+
+namespace trn {
+
+typedef _Float16 half_t;
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t uint2_t __attribute__((ext_vector_type(2)));
+typedef uint32_t uint4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kWave = 64;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// D(32x32) += A(32x16) * B(16x32), fp16 in, fp32 out.  Lane l supplies A[l%32][8*(l/32)..+7]
+// and B[8*(l/32)..+7][l%32]; it receives D[8*(r/4) + 4*(l/32) + r%4][l%32] in element r.
+__device__ __forceinline__ float16_t mfma32(half8_t a, half8_t b, float16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+// Combine a value with the one held by the lane 32 away (the other half of a 32x32 accumulator
+// column).  ds_bpermute-based exchange; used once per KV tile, so its cost is noise.
+// (v_permlane32_swap with both operands equal is folded by the compiler as if its two results were
+// the same value, which they are not -- do not use it for this.)
+__device__ __forceinline__ float half_max(float x) { return fmaxf(x, __shfl_xor(x, 32, 64)); }
+__device__ __forceinline__ float half_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+
+// Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane a points at 4 fp16
+// (8 bytes); lanes 4r..4r+3 together supply "row" r = 16 consecutive elements (their addresses need
+// not be adjacent in memory, only their order matters).  Lane i of the group receives element i of
+// rows 0..3.  With a row-major [k][n] tile in LDS this hands every lane 4 consecutive k for one n,
+// i.e. an MFMA operand whose contraction index runs down the tile's rows.
+typedef __fp16 fp16x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4_t lds_read_tr16(const half_t* p) {
+    fp16x4_t r = __builtin_amdgcn_ds_read_tr16_b64_v4f16(
+        (fp16x4_t __attribute__((address_space(3)))*)(p));
+    return __builtin_bit_cast(half4_t, r);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+__device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
+
+__device__ __forceinline__ uint32_t pack_half2(float a, float b) {
+    half2_t h = {(half_t)a, (half_t)b};
+    return __builtin_bit_cast(uint32_t, h);
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool pitch16(int64_t elems, int elem_bytes) { return ((elems * elem_bytes) & 15) == 0; }
+
+}  // namespace trn

@@ -1,0 +1,124 @@
+"""Operator-level wrappers over the C ABI: argument checks that raise Python exceptions
+(so a caller's `try/except` around `forward` behaves as with the reference's generated
+modules, vanilla_llama_benchmark.py:303-332), pointer/stride extraction, stream lookup.
+
+Every function writes into caller-owned tensors, launches on torch's current stream and
+returns None.  Nothing here allocates device memory.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev_half(t: torch.Tensor, name: str) -> None:
+    _need(isinstance(t, torch.Tensor), f"{name}: expected a tensor")
+    _need(t.is_cuda, f"{name}: expected a GPU tensor, got {t.device}")
+    _need(t.dtype == torch.float16, f"{name}: expected float16, got {t.dtype}")
+    _need(t.dim() == 0 or t.stride(-1) == 1, f"{name}: innermost stride must be 1")
+
+
+def _dev_float(t: torch.Tensor, name: str) -> None:
+    _need(isinstance(t, torch.Tensor) and t.is_cuda, f"{name}: expected a GPU tensor")
+    _need(t.dtype == torch.float32, f"{name}: expected float32, got {t.dtype}")
+    _need(t.stride(-1) == 1, f"{name}: innermost stride must be 1")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(t: torch.Tensor):
+    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+
+
+def rmsnorm(x: torch.Tensor, gamma: Optional[torch.Tensor], y: torch.Tensor, eps: float) -> None:
+    """y = RMSNorm(x) over the last axis; x, y [rows, cols] (row stride free), gamma [cols] or None."""
+    _dev_half(x, "x"); _dev_half(y, "y")
+    _need(x.dim() == 2 and y.shape == x.shape, f"x {tuple(x.shape)} / y {tuple(y.shape)}: expected equal 2-D shapes")
+    if gamma is not None:
+        _dev_half(gamma, "gamma")
+        _need(gamma.shape == (x.shape[1],), f"gamma {tuple(gamma.shape)}: expected ({x.shape[1]},)")
+    lib = _lib.load()
+    st = lib.trn_rmsnorm_f16(_ptr(x), _ptr(gamma), _ptr(y), 1, x.shape[0], x.shape[1],
+                             0, x.stride(0), 0, y.stride(0), 0, float(eps), _stream(x))
+    _lib.check("trn_rmsnorm_f16", st)
+
+
+def head_rmsnorm(x: torch.Tensor, gamma: Optional[torch.Tensor], y: torch.Tensor, eps: float,
+                 row_start: int = 0) -> None:
+    """Per-head RMSNorm over head_dim of rows [row_start:] of x [heads, seq, head_dim]
+    (heads may be a flattened batch*heads axis); other rows of y are left untouched."""
+    _dev_half(x, "x"); _dev_half(y, "y")
+    _need(x.dim() == 3 and y.shape == x.shape, "x, y: expected equal [heads, seq, head_dim] shapes")
+    _need(0 <= row_start <= x.shape[1], "row_start out of range")
+    if gamma is not None:
+        _dev_half(gamma, "gamma")
+        _need(gamma.shape == (x.shape[2],), "gamma: expected (head_dim,)")
+    lib = _lib.load()
+    st = lib.trn_rmsnorm_f16(_ptr(x), _ptr(gamma), _ptr(y), x.shape[0], x.shape[1] - row_start, x.shape[2],
+                             x.stride(0), x.stride(1), y.stride(0), y.stride(1), row_start, float(eps),
+                             _stream(x))
+    _lib.check("trn_rmsnorm_f16", st)
+
+
+def _attn_desc(q, k, v, o, scale, causal, q_norm, q_eps, noise, tau) -> _lib.AttnDesc:
+    for t, n in ((q, "q"), (k, "k")):
+        _dev_half(t, n)
+        _need(t.dim() == 4, f"{n}: expected [batch, heads, seq, head_dim], got {tuple(t.shape)}")
+    B, Hq, Sq, D = q.shape
+    _need(k.shape[0] == B and k.shape[3] == D, f"k {tuple(k.shape)} does not match q {tuple(q.shape)}")
+    Hkv, Skv = k.shape[1], k.shape[2]
+    d = _lib.AttnDesc()
+    d.batch, d.n_q_heads, d.n_kv_heads, d.seq_q, d.seq_kv, d.head_dim = B, Hq, Hkv, Sq, Skv, D
+    d.q_stride_b, d.q_stride_h, d.q_stride_s = q.stride(0), q.stride(1), q.stride(2)
+    d.k_stride_b, d.k_stride_h, d.k_stride_s = k.stride(0), k.stride(1), k.stride(2)
+    if v is not None:
+        _dev_half(v, "v"); _dev_half(o, "o")
+        _need(v.shape == k.shape, f"v {tuple(v.shape)} must equal k {tuple(k.shape)}")
+        _need(o.shape == q.shape, f"o {tuple(o.shape)} must equal q {tuple(q.shape)}")
+        d.v_stride_b, d.v_stride_h, d.v_stride_s = v.stride(0), v.stride(1), v.stride(2)
+        d.o_stride_b, d.o_stride_h, d.o_stride_s = o.stride(0), o.stride(1), o.stride(2)
+    d.scale, d.causal = float(scale), int(bool(causal))
+    d.q_norm, d.q_norm_eps = int(bool(q_norm)), float(q_eps)
+    if noise is not None:
+        _dev_float(noise, "noise")
+        _need(tuple(noise.shape) == (B, Hq, Sq, Skv), f"noise {tuple(noise.shape)}: expected {(B, Hq, Sq, Skv)}")
+        d.noise_stride_b, d.noise_stride_h, d.noise_stride_s = noise.stride(0), noise.stride(1), noise.stride(2)
+    d.tau = float(tau)
+    return d
+
+
+def _row_stat(t: Optional[torch.Tensor], name: str, shape) -> None:
+    if t is None:
+        return
+    _dev_float(t, name)
+    _need(tuple(t.shape) == tuple(shape) and t.is_contiguous(), f"{name}: expected contiguous float32 {tuple(shape)}")
+
+
+def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor] = None,
+              q_norm: bool = False, gamma_q: Optional[torch.Tensor] = None, q_eps: float = 0.0,
+              noise: Optional[torch.Tensor] = None, tau: float = 1.0,
+              lse_pert: Optional[torch.Tensor] = None) -> None:
+    """o = softmax(scale * q k^T [+causal]) v.  q,o [B,Hq,Sq,D]; k,v [B,Hkv,Skv,D] (strided views allowed).
+    Optional outputs: lse [B,Hq,Sq] fp32; with noise [B,Hq,Sq,Skv] fp32 also lse_pert."""
+    d = _attn_desc(q, k, v, o, scale, causal, q_norm, q_eps, noise, tau)
+    B, Hq, Sq, _ = q.shape
+    _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq))
+    if gamma_q is not None:
+        _dev_half(gamma_q, "gamma_q")
+        _need(gamma_q.shape == (q.shape[3],), "gamma_q: expected (head_dim,)")
+    _need(noise is None or lse_pert is not None, "noise given without lse_pert")
+    lib = _lib.load()
+    st = lib.trn_attn_fwd_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
+                              _ptr(noise), _ptr(lse_pert), _stream(q))
+    _lib.check("trn_attn_fwd_f16", st)
