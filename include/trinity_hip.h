@@ -115,10 +115,11 @@ int trn_attn_fwd_f16(const trn_attn_desc* desc, const void* q, const void* k, co
  *                   summed over queries as the generated kernel's C_out is,
  *                   keyformer_llama_benchmark.py:79)
  * out_sum, out_sumsq (nullable): float [batch, n_q_heads, seq_kv] contiguous.  Deterministic
- * (one workgroup owns a column block; no atomics).  v/o strides of desc are ignored.
+ * (one workgroup owns a column block; no atomics).  v/o strides of desc are ignored; desc->q_norm
+ * must be 0 (TRN_E_UNSUPPORTED otherwise).
  */
 int trn_attn_colstats_f16(const trn_attn_desc* desc, const void* q, const void* k,
-                          const float* lse, const void* gamma_q, const float* noise,
+                          const float* lse, const float* noise,
                           float* out_sum, float* out_sumsq, void* stream);
 
 /*

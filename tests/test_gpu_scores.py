@@ -1,0 +1,84 @@
+"""GPU parity for the key-score paths: forward (row LSE) + trn_attn_colstats_f16, against the CPU oracle.
+fp32 key scores: 1e-3 relative (plus 1e-5 absolute for near-zero columns)."""
+import pytest
+import torch
+
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+
+def close_scores(got, want, rtol=1e-3, atol=1e-5):
+    got = got.float().cpu(); want = want.float()
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bad.any(), f"{int(bad.sum())} off; max rel {(err / want.abs().clamp(min=1e-6)).max():.3g}"
+
+
+def make(B, Hq, Hkv, Sq, Skv, D, seed=42):
+    g = torch.Generator().manual_seed(seed)
+    return (ref.randn_half((B, Hq, Sq, D), g), ref.randn_half((B, Hkv, Skv, D), g), ref.randn_half((B, Hkv, Skv, D), g))
+
+
+def run_roco(q, k, v, scale, causal):
+    from triton_amd import ops
+    B, Hq, Sq, D = q.shape; Skv = k.shape[2]
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda")
+    s1 = torch.full((B, Hq, Skv), -1.0, device="cuda"); s2 = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, causal, lse=lse)
+    ops.attention_colstats(qd, kd, lse, scale, causal, s1, s2)
+    torch.cuda.synchronize()
+    return o, s1, s2
+
+
+CASES = [(1, 4, 2, 256, 256, 128, True), (1, 4, 2, 256, 256, 128, False), (2, 3, 1, 200, 200, 64, True),
+         (1, 2, 2, 16, 1040, 128, False), (1, 2, 2, 16, 1040, 64, True), (1, 8, 2, 640, 640, 128, True),
+         (1, 1, 1, 1, 1, 64, True), (1, 2, 1, 130, 259, 128, True)]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", CASES)
+def test_roco_parity(B, Hq, Hkv, Sq, Skv, D, causal):
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D)
+    scale = D ** -0.5
+    o, s1, s2 = run_roco(q, k, v, scale, causal)
+    wo, w1, w2 = ref.roco(q, k, v, scale, causal)
+    close_scores(s1, w1); close_scores(s2, w2)
+    assert (o.float().cpu() - wo.float()).abs().max() < 2e-2
+    # invariant: every row sums to 1, so the column sums add up to the number of queries
+    assert torch.allclose(s1.sum(-1).cpu(), torch.full((B, Hq), float(Sq)), rtol=1e-4)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,tau", [
+    (1, 4, 2, 256, 256, 128, True, 1.0), (1, 4, 2, 200, 200, 128, True, 1.5), (1, 3, 1, 96, 96, 64, False, 1.0),
+    (1, 2, 2, 16, 1040, 128, False, 1.5), (1, 2, 1, 130, 260, 64, True, 1.0)])
+def test_keyformer_parity(B, Hq, Hkv, Sq, Skv, D, causal, tau):
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=7)
+    noise = ref.gumbel_noise((B, Hq, Sq, Skv), 1234)
+    scale = D ** -0.5
+    qd, kd, vd, nd = q.cuda(), k.cuda(), v.cuda(), noise.cuda()
+    o = torch.zeros_like(qd); lsep = torch.zeros(B, Hq, Sq, device="cuda")
+    score = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, causal, noise=nd, tau=tau, lse_pert=lsep)
+    ops.attention_colstats(qd, kd, lsep, scale, causal, score, None, noise=nd, tau=tau)
+    torch.cuda.synchronize()
+    wo, wscore = ref.keyformer(q, k, v, noise, scale, tau, causal)
+    close_scores(score, wscore)
+    assert (o.float().cpu() - wo.float()).abs().max() < 2e-2
+    assert torch.allclose(score.sum(-1).cpu(), torch.full((B, Hq), float(Sq)), rtol=1e-4)
+
+
+def test_uniform_attention_harmonic_closed_form_on_gpu():
+    S, D = 300, 128
+    q, k, v = make(1, 2, 1, S, S, D, seed=3)
+    o, s1, s2 = run_roco(torch.zeros_like(q), k, v, 1.0, True)
+    want1 = ref.harmonic_tail(S, 1).float(); want2 = ref.harmonic_tail(S, 2).float()
+    close_scores(s1[0, 0], want1, rtol=1e-4); close_scores(s2[0, 1], want2, rtol=1e-4)
+
+
+def test_colstats_deterministic():
+    q, k, v = make(1, 4, 2, 384, 384, 128, seed=5)
+    _, a1, a2 = run_roco(q, k, v, 0.088, True)
+    _, b1, b2 = run_roco(q, k, v, 0.088, True)
+    assert torch.equal(a1, b1) and torch.equal(a2, b2)

@@ -69,7 +69,7 @@ def load() -> C.CDLL:
     lib.trn_attn_fwd_f16.restype = C.c_int
     lib.trn_attn_fwd_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.trn_attn_colstats_f16.restype = C.c_int
-    lib.trn_attn_colstats_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.trn_attn_colstats_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp]
     lib.trn_prenorm_qkv_f16.restype = C.c_int
     lib.trn_prenorm_qkv_f16.argtypes = [vp] * 8 + [i64] * 15 + [f32, i32, vp]
     _lib = lib

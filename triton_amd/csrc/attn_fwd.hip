@@ -266,6 +266,7 @@ static hipError_t launch_fwd(const AttnArgs& a, hipStream_t s) {
     return hipGetLastError();
 }
 
+int validate_attn(const trn_attn_desc* d, bool need_v);
 int validate_attn(const trn_attn_desc* d, bool need_v) {
     if (d->batch <= 0 || d->n_q_heads <= 0 || d->n_kv_heads <= 0 || d->seq_q <= 0 || d->seq_kv <= 0) return TRN_E_SHAPE;
     if (d->n_q_heads % d->n_kv_heads != 0) return TRN_E_SHAPE;

@@ -122,3 +122,22 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
     st = lib.trn_attn_fwd_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
                               _ptr(noise), _ptr(lse_pert), _stream(q))
     _lib.check("trn_attn_fwd_f16", st)
+
+
+def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
+                       out_sumsq: Optional[torch.Tensor] = None, noise: Optional[torch.Tensor] = None,
+                       tau: float = 1.0) -> None:
+    """Column sums (and sums of squares) of exp(t - lse) over the queries that see each key.
+    lse [B,Hq,Sq] is the row normaliser matching t (plain, or perturbed when noise is given).
+    out_sum / out_sumsq: float32 [B,Hq,Skv]."""
+    d = _attn_desc(q, k, None, None, scale, causal, False, 0.0, noise, tau)
+    B, Hq, Sq, _ = q.shape
+    Skv = k.shape[2]
+    _need(lse is not None, "lse is required")
+    _row_stat(lse, "lse", (B, Hq, Sq))
+    _row_stat(out_sum, "out_sum", (B, Hq, Skv)); _row_stat(out_sumsq, "out_sumsq", (B, Hq, Skv))
+    _need(out_sum is not None or out_sumsq is not None, "no output given")
+    lib = _lib.load()
+    st = lib.trn_attn_colstats_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(lse), _ptr(noise), _ptr(out_sum),
+                                   _ptr(out_sumsq), _stream(q))
+    _lib.check("trn_attn_colstats_f16", st)
