@@ -141,3 +141,32 @@ def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[
     st = lib.trn_attn_colstats_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(lse), _ptr(noise), _ptr(out_sum),
                                    _ptr(out_sumsq), _stream(q))
     _lib.check("trn_attn_colstats_f16", st)
+
+
+def prenorm_qkv(x: torch.Tensor, gamma: Optional[torch.Tensor], wq, wk, wv, q_out, k_out, v_out,
+                eps: float, norm: bool = True) -> None:
+    """Q,K,V = RMSNorm(x; gamma, eps) @ W{q,k,v}  (norm=False: x @ W).
+    x [T, hidden]; w* [hidden, n_*]; *_out indexed [head, token, head_dim] (any view with unit
+    innermost stride: a permuted token-major buffer, a head-major buffer, or rows of a KV cache)."""
+    _dev_half(x, "x")
+    _need(x.dim() == 2, "x: expected [tokens, hidden]")
+    T, K = x.shape
+    for w, n in ((wq, "wq"), (wk, "wk"), (wv, "wv")):
+        _dev_half(w, n)
+        _need(w.dim() == 2 and w.shape[0] == K, f"{n}: expected [hidden={K}, n_out], got {tuple(w.shape)}")
+    _need(wk.shape[1] == wv.shape[1], "wk and wv must have the same number of columns")
+    D = q_out.shape[-1]
+    for o, w, n in ((q_out, wq, "q_out"), (k_out, wk, "k_out"), (v_out, wv, "v_out")):
+        _dev_half(o, n)
+        _need(o.dim() == 3 and o.shape[1] == T and o.shape[2] == D and o.shape[0] * D == w.shape[1],
+              f"{n}: expected [heads, {T}, {D}] with heads*{D} == {w.shape[1]}, got {tuple(o.shape)}")
+    if gamma is not None:
+        _dev_half(gamma, "gamma")
+        _need(gamma.shape == (K,), "gamma: expected (hidden,)")
+    lib = _lib.load()
+    st = lib.trn_prenorm_qkv_f16(_ptr(x), _ptr(gamma), _ptr(wq), _ptr(wk), _ptr(wv), _ptr(q_out), _ptr(k_out),
+                                 _ptr(v_out), T, K, wq.shape[1], wk.shape[1], D, x.stride(0), wq.stride(0),
+                                 wk.stride(0), wv.stride(0), q_out.stride(0), q_out.stride(1), k_out.stride(0),
+                                 k_out.stride(1), v_out.stride(0), v_out.stride(1), float(eps), int(bool(norm)),
+                                 _stream(x))
+    _lib.check("trn_prenorm_qkv_f16", st)
