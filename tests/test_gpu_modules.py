@@ -1,0 +1,193 @@
+"""The drop-in boundary on the GPU: each FusedModule is driven exactly as the reference's
+benchmark_kernel drives a generated module (vanilla_llama_benchmark.py:243-291) -- positional
+tensors in TENSOR_PARAMS order, one eager call, warm-ups on a side stream, capture into a graph,
+replays -- and the tensors it leaves behind are compared with the CPU oracle."""
+import pytest
+import torch
+
+from oracle import ref
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want, atol=2e-2, rtol=1e-2):
+    got = got.float().cpu(); want = want.float()
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bad.any(), f"{int(bad.sum())} off; max abs err {err.max():.4g}"
+
+
+def drive(module, tensors, outputs, replays=3):
+    """The reference driver's call sequence.  Returns after the last replay has finished."""
+    args = [tensors[p] for p in module.TENSOR_PARAMS]
+    module.forward(*args)                                   # cold call
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(2):
+            module.forward(*args)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            module.forward(*args)
+    stream.synchronize()
+    for name in outputs:                                    # replays must regenerate the outputs
+        tensors[name].zero_()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        for _ in range(replays):
+            graph.replay()
+    stream.synchronize()
+
+
+def test_protocol_attributes_and_block_arguments():
+    from triton_amd import modules
+    from triton_amd.modules import vanilla
+    assert vanilla.TENSOR_PARAMS == sorted(vanilla.TENSOR_PARAMS) and vanilla.BLOCK_PARAMS == []
+    m = modules.get("vanilla")
+    g = torch.Generator().manual_seed(0)
+    q = ref.randn_half((2, 64, 64), g); k = ref.randn_half((1, 64, 64), g); v = ref.randn_half((1, 64, 64), g)
+    t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda())
+    args = [t[p] for p in m.TENSOR_PARAMS]
+    m.forward(*args, 32, 64)                     # block sizes positionally after the tensors
+    m.forward(*args, block_k=32, block_p=16)     # or as keywords
+    torch.cuda.synchronize()
+    close(t["O"], ref.attention(q[None], k[None], v[None], 64 ** -0.5, True)[0])
+    with pytest.raises(TypeError):
+        m.forward(*args[:-1])
+    with pytest.raises(TypeError):
+        m.forward(*args, foo=1)
+
+
+def test_prefill_modules_under_graph_replay():
+    from triton_amd import modules
+    g = torch.Generator().manual_seed(42)
+    B, Hq, Hkv, S, D = 1, 8, 2, 320, 128
+    q = ref.randn_half((B, Hq, S, D), g); k = ref.randn_half((B, Hkv, S, D), g); v = ref.randn_half((B, Hkv, S, D), g)
+    scale = D ** -0.5
+    dev = lambda t: t.cuda()
+    # vanilla
+    t = dict(Q=dev(q), K=dev(k), V=dev(v), O=torch.zeros_like(q).cuda())
+    drive(modules.get("vanilla"), t, ["O"])
+    want_o = ref.attention(q, k, v, scale, True)
+    close(t["O"], want_o)
+    # roco (fp32 outputs)
+    t = dict(Q=dev(q), K=dev(k), V=dev(v), O=torch.zeros_like(q).cuda(),
+             C_out1=torch.zeros(B, Hq, S, device="cuda"), C_out2=torch.zeros(B, Hq, S, device="cuda"))
+    drive(modules.get("roco"), t, ["O", "C_out1", "C_out2"])
+    _, s1, s2 = ref.roco(q, k, v, scale, True)
+    close(t["O"], want_o); close(t["C_out1"], s1, 1e-5, 1e-3); close(t["C_out2"], s2, 1e-5, 1e-3)
+    mean, std = modules.roco_mean_std(t["C_out1"], t["C_out2"], S, True)
+    wm, ws = ref.roco_mean_std(s1, s2, S, True)
+    close(mean, wm, 1e-6, 1e-3); close(std, ws, 1e-5, 5e-3)
+    # keyformer
+    noise = ref.gumbel_noise((B, Hq, S, S), 1234)
+    t = dict(Q=dev(q), K=dev(k), V=dev(v), O=torch.zeros_like(q).cuda(), noise=dev(noise),
+             C_out=torch.zeros(B, Hq, S, device="cuda"))
+    drive(modules.get("keyformer", tau=1.0), t, ["O", "C_out"])
+    _, sc = ref.keyformer(q, k, v, noise, scale, 1.0, True)
+    close(t["O"], want_o); close(t["C_out"], sc, 1e-5, 1e-3)
+
+
+def test_qknorm_and_rms_modules():
+    from triton_amd import modules
+    g = torch.Generator().manual_seed(3)
+    B, Hq, S, D = 1, 7, 200, 64
+    q = ref.randn_half((B, Hq, S, D), g); k = ref.randn_half((B, 1, S, D), g); v = ref.randn_half((B, 1, S, D), g)
+    gq = ref.randn_half((D,), g, 1, 0.02); gk = ref.randn_half((D,), g, 1, 0.02)
+    t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda(), gamma_q=gq.cuda(), gamma_k=gk.cuda())
+    drive(modules.get("qknorm", eps=1e-5), t, ["O"])
+    close(t["O"], ref.qknorm_attention(q, k, v, gq, gk, 1e-5, D ** -0.5, True))
+    x = ref.randn_half((300, 1024), g); gamma = ref.randn_half((1024,), g, 1, 0.02)
+    t = dict(X=x.cuda(), gamma=gamma.cuda(), X_norm=torch.zeros_like(x).cuda())
+    drive(modules.get("rms", eps=1e-5), t, ["X_norm"])
+    close(t["X_norm"], ref.rmsnorm(x, gamma, 1e-5), 1e-6, 1e-3)
+
+
+def test_prenorm_block_module():
+    from triton_amd import modules
+    g = torch.Generator().manual_seed(5)
+    B, S, N, D, Hkv = 1, 384, 1024, 128, 2
+    x = ref.randn_half((B, S, N), g); gamma = ref.randn_half((N,), g, 1, 0.02)
+    wq = ref.randn_half((N, N), g, 0, 0.02); wk = ref.randn_half((N, Hkv * D), g, 0, 0.02); wv = ref.randn_half((N, Hkv * D), g, 0, 0.02)
+    t = dict(X=x.cuda(), gamma=gamma.cuda(), WQ=wq.cuda(), WK=wk.cuda(), WV=wv.cuda(), O=torch.zeros(B, S, N, dtype=torch.float16, device="cuda"))
+    drive(modules.get("prenorm", head_dim=D, eps=1e-5), t, ["O"])
+    close(t["O"], ref.prenorm_block(x, gamma, wq, wk, wv, D, 1e-5, D ** -0.5, True))
+
+
+def _decode_tensors(M, N, D, P, seed=42, amp=1.0):
+    """The reference's input recipe (convert_eval_rms.py:170-201), scaled by `amp` where noted."""
+    H = N // D
+    g = torch.Generator().manual_seed(seed)
+    t = dict(X=ref.reference_recipe((M, N), g) * amp, WQ=ref.reference_recipe((N, N), g) * amp,
+             WK=ref.reference_recipe((N, N), g) * amp, WV=ref.reference_recipe((N, N), g) * amp,
+             K_cache=ref.reference_recipe((H, P + M, D), g) * amp, V_cache=ref.reference_recipe((H, P + M, D), g) * amp)
+    t["noise"] = torch.randn(H, M, P + M, generator=g).half()
+    return {k: v.half() for k, v in t.items()}, H
+
+
+@pytest.mark.parametrize("amp", [1.0, 30.0])
+def test_decode_append_modules_match_reference_classes(amp):
+    """Reference-faithful mode: scale 1, no mask, MHA, M=16 new tokens on a P-token cache."""
+    from triton_amd import modules
+    M, N, D, P = 16, 1024, 128, 200
+    cpu, H = _decode_tensors(M, N, D, P, amp=amp)
+    W = (cpu["WQ"], cpu["WK"], cpu["WV"])
+    atol = 2e-2 if amp > 1 else 1e-4
+
+    def fresh():
+        t = {k: v.cuda() for k, v in cpu.items()}
+        t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        return t
+
+    t = fresh()
+    drive(modules.get("vanilla", "decode", head_dim=D), t, ["O2"])
+    want = ref.decode_append_vanilla(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)
+    close(t["O2"], ref.flatten_token_major(want), atol)
+    q, k, v = ref._decode_qkv(cpu["X"], *W, D, False)
+    close(t["K_cache"][:, P:], k, atol); close(t["V_cache"][:, P:], v, atol)
+    assert torch.equal(t["K_cache"][:, :P].cpu(), cpu["K_cache"][:, :P])
+
+    # PreNorm makes |X_norm| ~ 1 whatever X's amplitude, so with amp=30 weights the unscaled scores reach
+    # the hundreds and the softmax amplifies fp16 rounding of q,k beyond any fixed tolerance; keep the
+    # weights at a tenth of that for this variant.
+    t = fresh()
+    wsc = 0.1 if amp > 1 else 1.0
+    for n in ("WQ", "WK", "WV"):
+        t[n] = (cpu[n] * wsc).half().cuda()
+    Wp = tuple((w * wsc).half() for w in W)
+    drive(modules.get("prenorm", "decode", head_dim=D), t, ["O2"])
+    close(t["O2"], ref.flatten_token_major(ref.decode_append_vanilla(cpu["X"], *Wp, cpu["K_cache"], cpu["V_cache"], P, D, prenorm=True)), atol)
+
+    t = fresh()
+    drive(modules.get("qknorm", "decode", head_dim=D), t, ["O2"])
+    close(t["O2"], ref.flatten_token_major(ref.decode_append_qknorm(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)), atol)
+
+    t = fresh(); t["C_out"] = torch.zeros(H, P + M, dtype=torch.float16, device="cuda")     # fp16 as the reference allocates it
+    drive(modules.get("keyformer", "decode", head_dim=D), t, ["O2", "C_out"])
+    wo, pw = ref.decode_append_keyformer(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], cpu["noise"], P, D, tau=1.5)
+    close(t["O2"], ref.flatten_token_major(wo), atol)
+    close(t["C_out"], pw.sum(dim=1), 1e-4, 5e-3 if amp > 1 else 2e-3)   # fp16 destination; see note on amp below
+
+    t = fresh(); t["C_out1"] = torch.zeros(H, P + M, device="cuda"); t["C_out2"] = torch.zeros(H, P + M, device="cuda")
+    drive(modules.get("roco", "decode", head_dim=D), t, ["O2", "C_out1", "C_out2"])
+    wo, s1, s2 = ref.decode_append_roco(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)
+    # q,k reach the score kernels through an fp16-rounded GEMM whose summation order differs from the
+    # oracle's, so a few of them differ by one fp16 ulp; with amp=30 the unscaled softmax magnifies that
+    # beyond the 1e-3 that holds for identical q,k (tests/test_gpu_scores.py) -- allow 5e-3 there.
+    srt = 5e-3 if amp > 1 else 1e-3
+    close(t["O2"], ref.flatten_token_major(wo), atol); close(t["C_out1"], s1, 1e-6, srt); close(t["C_out2"], s2, 1e-8, srt)
+
+
+def test_first_call_inside_capture_is_refused():
+    from triton_amd import modules
+    m = modules.get("roco")
+    q = torch.zeros(1, 2, 64, 64, dtype=torch.float16, device="cuda")
+    t = dict(Q=q, K=q.clone(), V=q.clone(), O=q.clone(), C_out1=torch.zeros(1, 2, 64, device="cuda"), C_out2=torch.zeros(1, 2, 64, device="cuda"))
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with pytest.raises(RuntimeError):
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                m.forward(*[t[p] for p in m.TENSOR_PARAMS])

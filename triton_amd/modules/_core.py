@@ -1,0 +1,346 @@
+"""Hand-written counterparts of the reference's generated modules.
+
+The reference's code generator emits, per IR candidate, a Python module with three
+attributes (TritonGen.py:568-712):
+
+    TENSOR_PARAMS : sorted names of the tensors `forward` takes (intermediates that fuse away
+                    are not listed)
+    BLOCK_PARAMS  : sorted names of tunable block-size keyword arguments
+    forward(*tensors, block_x=16, ...) -> None : launches the kernels on the current stream and
+                    writes the outputs in place
+
+and its drivers call `forward(*[tensors[p] for p in TENSOR_PARAMS])`, first eagerly, then on a
+side stream, then under graph capture (vanilla_llama_benchmark.py:243-285), sometimes with the
+block sizes as keywords (rms_benchmark.py:252) or positionally after the tensors
+(convert_eval_rms.py:275-285).  A FusedModule is such an object with the kernels replaced by
+libtrinity_hip.so calls: tile shapes are compile-time choices of the HIP kernels, so
+BLOCK_PARAMS is empty and any block-size argument is accepted and ignored.
+
+Shape constants that the reference bakes in at code-generation time (M, N, D, H, P and this
+build's scale / causal / eps / tau knobs) are constructor arguments here; the tensor shapes
+themselves are read from the tensors on every call.
+
+`forward` allocates nothing after its first call for a given set of shapes: the few
+intermediates that do not fuse away (row normalisers, the projected Q of the decode-append
+form, an fp32 copy of fp16 noise) live in a per-module workspace cache filled on that first,
+eager call -- the call the reference's drivers make before capturing a graph.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from .. import ops
+
+
+class FusedModule:
+    """Base: the three-attribute protocol plus a shape-keyed workspace cache."""
+
+    TENSOR_PARAMS: List[str] = []
+    BLOCK_PARAMS: List[str] = []
+
+    def __init__(self) -> None:
+        self._ws: Dict[Tuple, torch.Tensor] = {}
+
+    def _workspace(self, name: str, shape, dtype, device) -> torch.Tensor:
+        key = (name, tuple(shape), dtype, str(device))
+        t = self._ws.get(key)
+        if t is None:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError(
+                    f"{type(self).__name__}.forward: first call for shapes {tuple(shape)} is inside a graph "
+                    "capture; call forward once eagerly first (as the reference's drivers do)")
+            t = torch.empty(shape, dtype=dtype, device=device)
+            self._ws[key] = t
+        return t
+
+    def _split(self, args, kwargs):
+        n = len(self.TENSOR_PARAMS)
+        if len(args) < n:
+            raise TypeError(f"forward expects tensors {self.TENSOR_PARAMS}, got {len(args)} positional arguments")
+        for k in kwargs:
+            if not k.startswith("block_"):
+                raise TypeError(f"forward got an unexpected keyword argument '{k}'")
+        return dict(zip(self.TENSOR_PARAMS, args[:n]))     # trailing positionals are block sizes: ignored
+
+    def forward(self, *args, **kwargs) -> None:
+        self._run(**self._split(args, kwargs))
+
+    __call__ = forward
+
+    def _run(self, **tensors) -> None:  # pragma: no cover - abstract
+        raise NotImplementedError
+
+
+def _as4(t: torch.Tensor, name: str) -> torch.Tensor:
+    """[H,S,D] -> [1,H,S,D]; 4-D passes through."""
+    if t.dim() == 3:
+        return t.unsqueeze(0)
+    if t.dim() != 4:
+        raise ValueError(f"{name}: expected [heads, seq, head_dim] or [batch, heads, seq, head_dim], got {tuple(t.shape)}")
+    return t
+
+
+def _scale(scale: Optional[float], head_dim: int) -> float:
+    return head_dim ** -0.5 if scale is None else float(scale)
+
+
+def _store_scores(dst: torch.Tensor, src32: torch.Tensor) -> None:
+    """Key scores are produced in fp32; a caller-owned fp16 tensor (the reference allocates every
+    tensor as fp16, vanilla_llama_benchmark.py:131-139) receives them rounded."""
+    if dst.data_ptr() != src32.data_ptr():
+        dst.copy_(src32.view(dst.shape))
+
+
+# ============================================================================ prefill form
+class RMSNorm(FusedModule):
+    """X_norm = RMSNorm(X) * gamma   (ref_attn.py:348-350; gamma=None, eps=0: ref_rms.py:102-103)."""
+    TENSOR_PARAMS = ["X", "X_norm", "gamma"]
+
+    def __init__(self, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+
+    def _run(self, X, X_norm, gamma):
+        ops.rmsnorm(X.view(-1, X.shape[-1]), gamma, X_norm.view(-1, X.shape[-1]), self.eps)
+
+
+class Attention(FusedModule):
+    """O = softmax(scale * Q K^T [+causal]) V with GQA/MQA (ref_rms.py:77-80, :1466-1473)."""
+    TENSOR_PARAMS = ["K", "O", "Q", "V"]
+
+    def __init__(self, scale: Optional[float] = None, causal: bool = True):
+        super().__init__()
+        self.scale, self.causal = scale, causal
+
+    def _run(self, K, O, Q, V):
+        q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
+        ops.attention(q, k, v, o, _scale(self.scale, q.shape[-1]), self.causal)
+
+
+class QKNormAttention(FusedModule):
+    """Per-head RMSNorm of Q and K over head_dim, then attention (ref_rms.py:217-228).
+    K is normalised once into a workspace (it is shared by every query head); the Q norm is
+    fused into the attention kernel's prologue."""
+    TENSOR_PARAMS = ["K", "O", "Q", "V", "gamma_k", "gamma_q"]
+
+    def __init__(self, scale: Optional[float] = None, causal: bool = True, eps: float = 1e-5):
+        super().__init__()
+        self.scale, self.causal, self.eps = scale, causal, eps
+
+    def _run(self, K, O, Q, V, gamma_k, gamma_q):
+        q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
+        if not k.is_contiguous():
+            raise ValueError("K: expected a contiguous tensor")
+        B, Hkv, Skv, D = k.shape
+        kn = self._workspace("k_norm", k.shape, k.dtype, k.device)
+        ops.head_rmsnorm(k.view(B * Hkv, Skv, D), gamma_k, kn.view(B * Hkv, Skv, D), self.eps)
+        ops.attention(q, kn, v, o, _scale(self.scale, D), self.causal, q_norm=True, gamma_q=gamma_q, q_eps=self.eps)
+
+
+class KeyFormerAttention(FusedModule):
+    """Attention plus key scores C_out[h,j] = sum_i softmax_i((scale*QK^T + noise)/tau)[j]
+    (ref_rms.py:171-176; reduced over queries as the generated kernel's C_out is,
+    keyformer_llama_benchmark.py:79).  Two launches: forward (+ perturbed row normaliser),
+    then the column-owner pass."""
+    TENSOR_PARAMS = ["C_out", "K", "O", "Q", "V", "noise"]
+
+    def __init__(self, scale: Optional[float] = None, causal: bool = True, tau: float = 1.0):
+        super().__init__()
+        self.scale, self.causal, self.tau = scale, causal, tau
+
+    def _run(self, C_out, K, O, Q, V, noise):
+        q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
+        B, Hq, Sq, D = q.shape
+        Skv = k.shape[2]
+        n4 = _as4(noise, "noise")
+        if n4.dtype != torch.float32:                    # the reference's noise is fp16 (convert_eval_rms.py:201)
+            n32 = self._workspace("noise32", n4.shape, torch.float32, n4.device)
+            n32.copy_(n4)
+            n4 = n32
+        lsep = self._workspace("lse_pert", (B, Hq, Sq), torch.float32, q.device)
+        score = C_out.view(B, Hq, Skv) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
+            self._workspace("score32", (B, Hq, Skv), torch.float32, q.device)
+        sc = _scale(self.scale, D)
+        ops.attention(q, k, v, o, sc, self.causal, noise=n4, tau=self.tau, lse_pert=lsep)
+        ops.attention_colstats(q, k, lsep, sc, self.causal, score, None, noise=n4, tau=self.tau)
+        _store_scores(C_out, score)
+
+
+class RoCoAttention(FusedModule):
+    """Attention plus per-key column sum C_out1 and column sum of squares C_out2 of the attention
+    probabilities (ref_rms.py:274-275).  mean/std are derived by roco_mean_std below."""
+    TENSOR_PARAMS = ["C_out1", "C_out2", "K", "O", "Q", "V"]
+
+    def __init__(self, scale: Optional[float] = None, causal: bool = True):
+        super().__init__()
+        self.scale, self.causal = scale, causal
+
+    def _run(self, C_out1, C_out2, K, O, Q, V):
+        q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
+        B, Hq, Sq, D = q.shape
+        Skv = k.shape[2]
+        lse = self._workspace("lse", (B, Hq, Sq), torch.float32, q.device)
+        outs = []
+        for i, c in enumerate((C_out1, C_out2)):
+            outs.append(c.view(B, Hq, Skv) if c.dtype == torch.float32 and c.is_contiguous() else
+                        self._workspace(f"stat32_{i}", (B, Hq, Skv), torch.float32, q.device))
+        sc = _scale(self.scale, D)
+        ops.attention(q, k, v, o, sc, self.causal, lse=lse)
+        ops.attention_colstats(q, k, lse, sc, self.causal, outs[0], outs[1])
+        _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
+
+
+def roco_mean_std(s1: torch.Tensor, s2: torch.Tensor, seq_q: int, causal: bool):
+    """Per-key mean and (population) standard deviation of the attention probabilities over the
+    queries that can see the key, from RoCo's two sums.  n_j = seq_q - max(0, j - (seq_kv - seq_q))
+    under a causal mask, seq_q otherwise.  The reference defines only the sums; this derived
+    convention is this build's own."""
+    skv = s1.shape[-1]
+    if causal:
+        j = torch.arange(skv, device=s1.device)
+        n = (seq_q - (j - (skv - seq_q)).clamp(min=0)).to(s1.dtype)
+    else:
+        n = torch.full((skv,), float(seq_q), device=s1.device, dtype=s1.dtype)
+    mean = s1 / n
+    return mean, (s2 / n - mean * mean).clamp(min=0).sqrt()
+
+
+class PreNormBlock(FusedModule):
+    """O = Attention(RMSNorm(X) Wq, RMSNorm(X) Wk, RMSNorm(X) Wv), token-major in and out
+    (ref_rms.py:101-127 with the layout of ref_rms.py:1477).  X [B,S,hidden], O [B,S,Hq*D].
+    Two launches: the RMSNorm-fused projection GEMM writes Q/K/V token-major into a workspace,
+    attention reads them as strided [B,H,S,D] views and writes O token-major."""
+    TENSOR_PARAMS = ["O", "WK", "WQ", "WV", "X", "gamma"]
+
+    def __init__(self, head_dim: int = 128, scale: Optional[float] = None, causal: bool = True,
+                 eps: float = 1e-5, norm: bool = True):
+        super().__init__()
+        self.head_dim, self.scale, self.causal, self.eps, self.norm = head_dim, scale, causal, eps, norm
+
+    def _run(self, O, WK, WQ, WV, X, gamma):
+        D = self.head_dim
+        x3 = X if X.dim() == 3 else X.unsqueeze(0)
+        o3 = O if O.dim() == 3 else O.unsqueeze(0)
+        B, S, K = x3.shape
+        nq, nkv = WQ.shape[1], WK.shape[1]
+        if not x3.is_contiguous() or not o3.is_contiguous():
+            raise ValueError("X, O: expected contiguous tensors")
+        qkv = self._workspace("qkv", (B * S, nq + 2 * nkv), X.dtype, X.device)
+        qb, kb, vb = qkv[:, :nq], qkv[:, nq:nq + nkv], qkv[:, nq + nkv:]
+        hm = lambda t, n: t.view(B * S, n // D, D).permute(1, 0, 2)          # [head, token, D] view
+        ops.prenorm_qkv(x3.view(B * S, K), gamma, WQ, WK, WV, hm(qb, nq), hm(kb, nkv), hm(vb, nkv), self.eps, self.norm)
+        b4 = lambda t, n: t.view(B, S, n // D, D).permute(0, 2, 1, 3)        # [B, H, S, D] view
+        ops.attention(b4(qb, nq), b4(kb, nkv), b4(vb, nkv), b4(o3, nq), _scale(self.scale, D), self.causal)
+
+
+# ============================================================================ decode-append form
+class _DecodeAppend(FusedModule):
+    """Common part of the reference's own problem form (ref_rms.py:45-83): M new tokens X [M,N] are
+    projected with WQ/WK/WV [N,N]; K and V rows are appended in place at rows P..P+M of the
+    [H,P+M,D] caches (convert_eval_rms.py:146-147); every query then attends to all P+M keys with
+    no mask and no scale; O2 [M,N] is token-major (convert_eval_rms.py:160)."""
+
+    def __init__(self, head_dim: int, prenorm: bool = False, scale: float = 1.0, causal: bool = False):
+        super().__init__()
+        self.head_dim, self.prenorm, self.scale, self.causal = head_dim, prenorm, scale, causal
+
+    def _project(self, X, WQ, WK, WV, K_cache, V_cache):
+        M, N = X.shape
+        D = self.head_dim
+        H, PM, _ = K_cache.shape
+        P = PM - M
+        if H * D != N or P < 0 or K_cache.shape != V_cache.shape or K_cache.shape[2] != D:
+            raise ValueError(f"inconsistent shapes: X {tuple(X.shape)}, caches {tuple(K_cache.shape)}, head_dim {D}")
+        q = self._workspace("q", (H, M, D), X.dtype, X.device)
+        ops.prenorm_qkv(X, None, WQ, WK, WV, q, K_cache[:, P:], V_cache[:, P:], 0.0, self.prenorm)
+        return q, P
+
+    @staticmethod
+    def _o_view(O2, H, M, D):
+        return O2.view(M, H, D).permute(1, 0, 2).unsqueeze(0)               # [1,H,M,D] view of token-major O2
+
+
+class DecodeVanilla(_DecodeAppend):
+    """Vanila.forward / PreNorm.forward (ref_rms.py:45-83 / 101-127)."""
+    TENSOR_PARAMS = ["K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X"]
+
+    def _run(self, K_cache, O2, V_cache, WK, WQ, WV, X):
+        q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
+        H, M, D = q.shape
+        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal)
+
+
+class DecodeQKNorm(_DecodeAppend):
+    """QKNorm.forward (ref_rms.py:197-231): q and the newly appended k rows are normalised
+    (no eps, no weight); the cached prefix is used as stored."""
+    TENSOR_PARAMS = ["K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X"]
+
+    def _run(self, K_cache, O2, V_cache, WK, WQ, WV, X):
+        q, P = self._project(X, WQ, WK, WV, K_cache, V_cache)
+        H, M, D = q.shape
+        ops.head_rmsnorm(K_cache, None, K_cache, 0.0, row_start=P)          # in place, rows P.. only
+        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
+                      q_norm=True, gamma_q=None, q_eps=0.0)
+
+
+class DecodeKeyFormer(_DecodeAppend):
+    """KeyFormer.forward (ref_rms.py:147-179) with the perturbed probabilities summed over the M
+    queries into C_out [H,P+M] as the generated kernel does (keyformer_llama_benchmark.py:79)."""
+    TENSOR_PARAMS = ["C_out", "K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X", "noise"]
+
+    def __init__(self, head_dim: int, tau: float = 1.5, **kw):
+        super().__init__(head_dim, **kw)
+        self.tau = tau
+
+    def _run(self, C_out, K_cache, O2, V_cache, WK, WQ, WV, X, noise):
+        q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
+        H, M, D = q.shape
+        PM = K_cache.shape[1]
+        n4 = noise[None]
+        if n4.dtype != torch.float32:
+            n32 = self._workspace("noise32", n4.shape, torch.float32, n4.device)
+            n32.copy_(n4)
+            n4 = n32
+        lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
+        score = C_out.view(1, H, PM) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
+            self._workspace("score32", (1, H, PM), torch.float32, X.device)
+        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
+                      noise=n4, tau=self.tau, lse_pert=lsep)
+        ops.attention_colstats(q[None], K_cache[None], lsep, self.scale, self.causal, score, None, noise=n4, tau=self.tau)
+        _store_scores(C_out, score)
+
+
+class DecodeRoCo(_DecodeAppend):
+    """RoCo.forward (ref_rms.py:249-280): C_out1 = weights.sum(dim=1), C_out2 = weights.pow(2).sum(dim=1)."""
+    TENSOR_PARAMS = ["C_out1", "C_out2", "K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X"]
+
+    def _run(self, C_out1, C_out2, K_cache, O2, V_cache, WK, WQ, WV, X):
+        q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
+        H, M, D = q.shape
+        PM = K_cache.shape[1]
+        lse = self._workspace("lse", (1, H, M), torch.float32, X.device)
+        outs = []
+        for i, c in enumerate((C_out1, C_out2)):
+            outs.append(c.view(1, H, PM) if c.dtype == torch.float32 and c.is_contiguous() else
+                        self._workspace(f"stat32_{i}", (1, H, PM), torch.float32, X.device))
+        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal, lse=lse)
+        ops.attention_colstats(q[None], K_cache[None], lse, self.scale, self.causal, outs[0], outs[1])
+        _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
+
+
+PREFILL = {"rms": RMSNorm, "vanilla": Attention, "prenorm": PreNormBlock, "qknorm": QKNormAttention,
+           "keyformer": KeyFormerAttention, "roco": RoCoAttention}
+DECODE = {"vanilla": DecodeVanilla, "prenorm": lambda **kw: DecodeVanilla(prenorm=True, **kw),
+          "qknorm": DecodeQKNorm, "keyformer": DecodeKeyFormer, "roco": DecodeRoCo}
+
+
+def get(variant: str, form: str = "prefill", **consts) -> FusedModule:
+    """Module for `variant` in {'rms','vanilla','prenorm','qknorm','keyformer','roco'}.
+    form='prefill': Q/K/V (or X and weights) given, causal, 1/sqrt(D) scale by default.
+    form='decode' : the reference's decode-append problem (needs head_dim=...)."""
+    table = PREFILL if form == "prefill" else DECODE if form == "decode" else None
+    if table is None or variant not in table:
+        raise KeyError(f"no module for variant={variant!r} form={form!r}")
+    return table[variant](**consts)
