@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload vanilla|all|...]
+
+A "step" is one `forward` of the vanilla causal GQA attention module on the Llama3-8B shape
+(batch 1, 32 query / 8 KV heads, seq 4096, head_dim 128, fp16): the configuration the headline
+metric is quoted on.  Inputs are synthetic, generated from a seed, and resident in HBM before the
+timed region.  Timing follows the reference's own method (vanilla_llama_benchmark.py:254-294): one
+cold call, warm-ups on a side stream, `forward` captured into a graph, K replays -- bracketed here
+by device synchronisation and a wall clock for `value`, and by events on the launch stream for the
+kernel's own duration (`roofline`).
+
+Prints ONE JSON line.  `value` = causal-halved attention flops (4*B*H*S^2*D/2) per second.  The same
+line carries the RMSNorm [4096x4096] HBM rate (rotating buffers, so the 256 MB last-level cache
+cannot serve the reads), the other variants' rates when --workload all, and the CPU oracle timed on
+this machine's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="default",
+                    help="default (vanilla headline + rmsnorm), all, or one of vanilla rmsnorm prenorm qknorm keyformer roco")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
+    return ap.parse_args()
+
+
+def graph_timed(module, tensors, steps, warmup):
+    """Reference driver sequence; returns (wall ms/step, event ms/step)."""
+    import torch
+    args = [tensors[p] for p in module.TENSOR_PARAMS]
+    module.forward(*args)                       # cold call (allocates the module's workspaces)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for _ in range(max(warmup, 1)):
+            module.forward(*args)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            module.forward(*args)
+    stream.synchronize()
+    with torch.cuda.stream(stream):             # graph warm-up
+        for _ in range(3):
+            graph.replay()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        start.record()
+        for _ in range(steps):
+            graph.replay()
+        end.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    return wall_ms, start.elapsed_time(end) / steps
+
+
+def rotating_timed(fn_for, n_buffers, steps, warmup):
+    """Eager launches cycling over n_buffers buffer sets; returns (wall ms/step, event ms/step)."""
+    import torch
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(max(warmup, n_buffers)):
+            fn_for(i % n_buffers)
+    stream.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(stream):
+        start.record()
+        for i in range(steps):
+            fn_for(i % n_buffers)
+        end.record()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps, start.elapsed_time(end) / steps
+
+
+def attn_inputs(cfg, seed=42):
+    import torch
+    from oracle import ref
+    g = torch.Generator().manual_seed(seed)
+    B, Hq, Hkv, S, D = cfg["batch"], cfg["n_heads"], cfg["n_kv_heads"], cfg["seq"], cfg["head_dim"]
+    q = ref.randn_half((B, Hq, S, D), g); k = ref.randn_half((B, Hkv, S, D), g); v = ref.randn_half((B, Hkv, S, D), g)
+    return q, k, v
+
+
+def bench_vanilla(steps, warmup):
+    import torch
+    from triton_amd import configs, modules
+    cfg = configs.VANILLA
+    q, k, v = attn_inputs(cfg)
+    t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda())
+    wall, ev = graph_timed(modules.get("vanilla"), t, steps, warmup)
+    flops = configs.attn_flops(cfg["batch"], cfg["n_heads"], cfg["seq"], cfg["seq"], cfg["head_dim"], True)
+    return dict(wall_ms=wall, kernel_ms=ev, flops=flops, tflops=flops / wall / 1e9, kernel_tflops=flops / ev / 1e9,
+                tensors=(q, k, v))
+
+
+def bench_rmsnorm(steps, warmup):
+    import torch
+    from triton_amd import configs, modules
+    cfg = configs.RMSNORM
+    R = 16                                            # 16 x (32 MiB in + 32 MiB out) = 1 GiB >> 256 MB cache
+    gen = torch.Generator(device="cuda").manual_seed(42)
+    xs = [torch.randn(cfg["rows"], cfg["cols"], device="cuda", generator=gen).half() for _ in range(R)]
+    ys = [torch.empty_like(x) for x in xs]
+    gamma = (1 + 0.02 * torch.randn(cfg["cols"], device="cuda", generator=gen)).half()
+    m = modules.get("rms", eps=cfg["eps"])
+    wall, ev = rotating_timed(lambda i: m.forward(xs[i], ys[i], gamma), R, max(steps, 64), warmup)
+    hot_wall, hot_ev = rotating_timed(lambda i: m.forward(xs[0], ys[0], gamma), 1, max(steps, 64), warmup)
+    nbytes = configs.rmsnorm_bytes(cfg["rows"], cfg["cols"])
+    return dict(kernel_us=ev * 1e3, gbps=nbytes / ev / 1e6, frac=nbytes / ev / 1e6 / configs.HBM_PEAK_GBPS,
+                hot_cache_gbps=nbytes / hot_ev / 1e6, bytes=nbytes, rotating_buffers=R)
+
+
+def bench_variant(name, steps, warmup):
+    import torch
+    from oracle import ref
+    from triton_amd import configs, modules
+    g = torch.Generator().manual_seed(42)
+    if name == "qknorm":
+        cfg = configs.QKNORM
+        q, k, v = attn_inputs(cfg)
+        D = cfg["head_dim"]
+        t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda(),
+                 gamma_q=ref.randn_half((D,), g, 1, 0.02).cuda(), gamma_k=ref.randn_half((D,), g, 1, 0.02).cuda())
+        m = modules.get("qknorm", eps=cfg["eps"])
+        flops = configs.attn_flops(1, cfg["n_heads"], cfg["seq"], cfg["seq"], D, True)
+    elif name == "prenorm":
+        cfg = configs.PRENORM
+        S, N, D = cfg["seq"], cfg["hidden"], cfg["head_dim"]
+        nkv = cfg["n_kv_heads"] * D
+        t = dict(X=ref.randn_half((1, S, N), g).cuda(), gamma=ref.randn_half((N,), g, 1, 0.02).cuda(),
+                 WQ=ref.randn_half((N, N), g, 0, 0.02).cuda(), WK=ref.randn_half((N, nkv), g, 0, 0.02).cuda(),
+                 WV=ref.randn_half((N, nkv), g, 0, 0.02).cuda(), O=torch.zeros(1, S, N, dtype=torch.float16, device="cuda"))
+        m = modules.get("prenorm", head_dim=D, eps=cfg["eps"])
+        flops = configs.qkv_gemm_flops(S, N, N, nkv) + configs.attn_flops(1, cfg["n_heads"], S, S, D, True)
+    elif name in ("keyformer", "roco"):
+        cfg = configs.KEYFORMER if name == "keyformer" else configs.ROCO
+        q, k, v = attn_inputs(cfg)
+        B, Hq, S, D = 1, cfg["n_heads"], cfg["seq"], cfg["head_dim"]
+        t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda())
+        if name == "keyformer":
+            gen = torch.Generator(device="cuda").manual_seed(cfg["noise_seed"])     # throughput only: device-side noise
+            u = torch.rand(B, Hq, S, S, device="cuda", generator=gen).clamp_(1e-10, 1 - 1e-7)
+            t["noise"] = -torch.log(-torch.log(u)); del u
+            t["C_out"] = torch.zeros(B, Hq, S, device="cuda")
+            m = modules.get("keyformer", tau=cfg["tau"])
+        else:
+            t["C_out1"] = torch.zeros(B, Hq, S, device="cuda"); t["C_out2"] = torch.zeros(B, Hq, S, device="cuda")
+            m = modules.get("roco")
+        flops = configs.attn_flops(1, Hq, S, S, D, True)
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    wall, ev = graph_timed(m, t, steps, warmup)
+    out = dict(ms=ev, tflops=flops / ev / 1e9, frac_mfma=flops / ev / 1e9 / configs.MFMA_F16_PEAK_TFLOPS)
+    if name == "keyformer":
+        S, Hq = cfg["seq"], cfg["n_heads"]
+        nbytes = Hq * S * (S + 1) // 2 * 4 + 83886080 + Hq * S * 4 * 4
+        out.update(algorithmic_bytes=nbytes, gbps=nbytes / ev / 1e6, frac_hbm=nbytes / ev / 1e6 / configs.HBM_PEAK_GBPS)
+    return out
+
+
+def cpu_baseline(q, k, v, budget_s):
+    """The CPU oracle (oracle/ref.py, eager PyTorch fp32 on the host cores) on a bounded sample of the
+    headline workload: whole query heads at the full S=4096, head by head, until the time budget is
+    spent.  Rate = causal-halved flops of the heads done / seconds."""
+    import torch
+    from oracle import ref
+    from triton_amd import configs
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cores = max(1, min(cores, int(os.environ.get("OMP_NUM_THREADS", cores))))
+    torch.set_num_threads(cores)
+    B, Hq, S, D = q.shape
+    G = Hq // k.shape[1]
+    scale = D ** -0.5
+    ref.attention(q[:, :1, :512], k[:, :1, :512], v[:, :1, :512], scale, True)       # warm-up
+    done, t0 = 0, time.perf_counter()
+    while done < Hq and (done == 0 or time.perf_counter() - t0 < budget_s):
+        h = done
+        ref.attention(q[:, h:h + 1], k[:, h // G:h // G + 1], v[:, h // G:h // G + 1], scale, True)
+        done += 1
+    dt = time.perf_counter() - t0
+    flops = configs.attn_flops(B, done, S, S, D, True)
+    return dict(value=flops / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                sample=f"{done} of {Hq} query heads at S={S}, D={D} (full rows, fp32 eager PyTorch), {dt:.1f} s")
+
+
+def main():
+    a = parse()
+    if a.gpus != 1:
+        print(f"bench.py measures one GPU only (got --gpus {a.gpus}): this build's hot path is single-GPU; "
+              "heads shard across GPUs without collectives, and no multi-GPU figure is produced.", file=sys.stderr)
+        raise SystemExit(2)
+    import torch
+    from triton_amd import _lib, configs
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU: there is no CPU fallback for the kernels")
+    _lib.check("trn_check_device", _lib.load().trn_check_device())
+
+    wl = a.workload
+    extra = {}
+    van = bench_vanilla(a.steps, a.warmup) if wl in ("default", "all", "vanilla") else None
+    if wl in ("default", "all", "rmsnorm"):
+        extra["rmsnorm"] = bench_rmsnorm(a.steps, a.warmup)
+    for name in ("prenorm", "qknorm", "keyformer", "roco"):
+        if wl in ("all", name):
+            extra[name] = bench_variant(name, max(a.steps // 4, 10), a.warmup)
+            torch.cuda.empty_cache()
+    if van is None:                       # a single non-headline workload was asked for
+        print(json.dumps({"workload": wl, **extra}))
+        return
+
+    peak = configs.MFMA_F16_PEAK_TFLOPS
+    line = {
+        "metric": "attn TFLOP/s + % fp16 MFMA peak (Llama3-8B, S=4096); RMSNorm HBM GB/s",
+        "value": round(van["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(van["wall_ms"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "vanilla causal GQA attention, batch 1, seq 4096, 32 q heads / 8 kv heads, head_dim 128",
+                   "flops_per_step": van["flops"], "flop_convention": "4*B*H*S^2*D/2 (causal-halved)",
+                   "timing": "graph replay on a side stream"},
+        "pct_of_fp16_mfma_peak": round(100 * van["tflops"] / peak, 2),
+        "roofline": {"bound": "mfma", "achieved": round(van["kernel_tflops"], 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(van["kernel_tflops"] / peak, 4), "traffic": None,
+                     "kernel": "attn_fwd_kernel<128>", "kernel_ms": round(van["kernel_ms"], 5)},
+    }
+    if "rmsnorm" in extra:
+        r = extra["rmsnorm"]
+        line["rmsnorm"] = {"value": round(r["gbps"], 1), "unit": "GB/s", "frac_of_hbm_peak": round(r["frac"], 4),
+                           "kernel_us": round(r["kernel_us"], 3), "bytes": r["bytes"],
+                           "rotating_buffers": r["rotating_buffers"], "cache_hot_gbps": round(r["hot_cache_gbps"], 1),
+                           "workload": "RMSNorm fp16 [4096 x 4096], gamma, eps 1e-5"}
+    for name in ("prenorm", "qknorm", "keyformer", "roco"):
+        if name in extra:
+            line[name] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in extra[name].items()}
+    if not a.no_cpu:
+        line["cpu_baseline"] = cpu_baseline(*van["tensors"], a.cpu_seconds)
+        line["cpu_baseline"]["value"] = round(line["cpu_baseline"]["value"], 4)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,153 @@
+"""CPU-side checks (no GPU, no compute calls): the C-ABI library loads and exports every symbol the
+header declares, the ctypes mirror of trn_attn_desc matches the C layout, argument validation that
+happens before any launch returns the documented status codes, and the module protocol's host logic."""
+import ctypes as C
+import os
+import re
+import subprocess
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "trinity_hip.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from triton_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from triton_amd import build
+        build.build(verbose=False)
+    return _lib.load()
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(trn_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    from triton_amd import _lib
+    names = declared_functions()
+    assert names, "no declarations parsed from the header"
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/trinity_hip.h but not exported"
+    assert sorted(_lib.EXPORTS) == names
+
+
+def test_version_and_status_names(lib):
+    assert lib.trn_version() >= 100
+    assert lib.trn_status_name(0) == b"TRN_OK"
+    assert lib.trn_status_name(-5) == b"TRN_E_UNSUPPORTED"
+    assert lib.trn_status_name(-99) == b"TRN_E_UNKNOWN"
+
+
+def test_attn_desc_layout_matches_c(tmp_path):
+    """Compile a tiny C program against the header and compare sizeof/offsetof with ctypes."""
+    from triton_amd._lib import AttnDesc
+    fields = [f[0] for f in AttnDesc._fields_]
+    src = tmp_path / "layout.c"
+    lines = ['#include <stdio.h>', '#include <stddef.h>', f'#include "{HEADER}"', 'int main(void){',
+             'printf("%zu\\n", sizeof(trn_attn_desc));']
+    lines += [f'printf("%zu\\n", offsetof(trn_attn_desc, {f}));' for f in fields]
+    lines += ['return 0;}']
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", str(src), "-o", str(exe)], check=True)
+    out = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    assert out[0] == C.sizeof(AttnDesc)
+    for f, off in zip(fields, out[1:]):
+        assert getattr(AttnDesc, f).offset == off, f
+
+
+def _desc(**kw):
+    from triton_amd._lib import AttnDesc
+    d = AttnDesc()
+    base = dict(batch=1, n_q_heads=4, n_kv_heads=2, seq_q=8, seq_kv=8, head_dim=64, scale=0.125, causal=1,
+                q_stride_b=2048, q_stride_h=512, q_stride_s=64, k_stride_b=1024, k_stride_h=512, k_stride_s=64,
+                v_stride_b=1024, v_stride_h=512, v_stride_s=64, o_stride_b=2048, o_stride_h=512, o_stride_s=64, tau=1.0)
+    base.update(kw)
+    for k, v in base.items():
+        setattr(d, k, v)
+    return d
+
+
+def test_validation_rejects_before_launch(lib):
+    """Every call below fails validation, so no kernel is launched and no device is touched."""
+    p = C.c_void_p(0x1000)       # non-null, 16-byte aligned dummy; never dereferenced on these paths
+    fwd = lambda d, q=p: lib.trn_attn_fwd_f16(C.byref(d), q, p, p, p, None, None, None, None, None)
+    assert fwd(_desc(), None) == -1                                   # TRN_E_NULL
+    assert fwd(_desc(head_dim=32)) == -5                              # TRN_E_UNSUPPORTED
+    assert fwd(_desc(n_q_heads=3)) == -2                              # heads not a multiple of kv heads
+    assert fwd(_desc(seq_kv=4)) == -2                                 # causal with fewer keys than queries
+    assert fwd(_desc(scale=0.0)) == -5
+    assert fwd(_desc(q_stride_s=32)) == -3                            # TRN_E_STRIDE
+    assert fwd(_desc(k_stride_h=516)) == -4                           # pitch not 16-byte aligned
+    assert fwd(_desc(), C.c_void_p(0x1008)) == -4                     # pointer not 16-byte aligned
+    assert lib.trn_attn_fwd_f16(C.byref(_desc()), p, p, p, p, None, None, p, None, None) == -1   # noise without lse_pert
+    assert lib.trn_attn_colstats_f16(C.byref(_desc()), p, p, p, None, None, None, None) == -1    # no output
+    assert lib.trn_attn_colstats_f16(C.byref(_desc(q_norm=1)), p, p, p, None, p, None, None) == -5
+    rms = lambda cols, ld, x=p: lib.trn_rmsnorm_f16(x, None, p, 1, 4, cols, 0, ld, 0, ld, 0, 0.0, None)
+    assert rms(12, 12) == -2 and rms(64, 32) == -3 and rms(64, 68) == -4 and rms(64, 64, None) == -1
+    assert lib.trn_rmsnorm_f16(None, None, None, 1, 0, 64, 0, 64, 0, 64, 0, 0.0, None) == 0      # zero rows: no-op
+    g = lambda **kw: lib.trn_prenorm_qkv_f16(p, None, p, p, p, p, p, p, *[kw.get(k, v) for k, v in dict(
+        tokens=16, hidden=64, n_q=64, n_kv=64, head_dim=64, ldx=64, ldwq=64, ldwk=64, ldwv=64, qh=64, qs=64, kh=64,
+        ks=64, vh=64, vs=64).items()], 0.0, 1, None)
+    assert g(hidden=60) == -2 and g(n_q=96) == -2 and g(ldx=32) == -3 and g(ldwq=68) == -4 and g(qs=32) == -3
+    assert g(tokens=0) == 0
+
+
+def test_wrappers_raise_python_exceptions_on_cpu_tensors():
+    from triton_amd import ops
+    x = torch.zeros(4, 64, dtype=torch.float16)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        ops.rmsnorm(x, None, x.clone(), 0.0)
+    q = torch.zeros(1, 2, 8, 64, dtype=torch.float16)
+    with pytest.raises(ValueError):
+        ops.attention(q, q, q, q, 1.0, True)
+
+
+def test_module_protocol_host_logic():
+    from triton_amd import modules
+    from triton_amd.modules import keyformer, prenorm, qknorm, rms, roco, vanilla
+    for mod in (keyformer, prenorm, qknorm, rms, roco, vanilla):
+        assert mod.TENSOR_PARAMS == sorted(mod.TENSOR_PARAMS, key=lambda s: s) and mod.BLOCK_PARAMS == []
+        assert callable(mod.forward)
+    # names the reference's drivers know (vanilla_llama_benchmark.py:42-77, keyformer_llama_benchmark.py:74-79)
+    assert modules.get("vanilla", "decode", head_dim=128).TENSOR_PARAMS == ["K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X"]
+    assert "noise" in modules.get("keyformer", "decode", head_dim=128).TENSOR_PARAMS
+    assert {"C_out1", "C_out2"} <= set(modules.get("roco", "decode", head_dim=64).TENSOR_PARAMS)
+    with pytest.raises(KeyError):
+        modules.get("nope")
+    m = modules.get("vanilla")
+    with pytest.raises(TypeError):
+        m.forward(torch.zeros(1))                       # too few tensors
+    s1 = torch.tensor([[2.0, 1.0, 0.5]]); s2 = torch.tensor([[1.5, 0.6, 0.25]])
+    mean, std = modules.roco_mean_std(s1, s2, 3, True)
+    assert torch.allclose(mean, torch.tensor([[2 / 3, 0.5, 0.5]]))
+    assert torch.allclose(std, (s2 / torch.tensor([3.0, 2.0, 1.0]) - mean ** 2).clamp(min=0).sqrt())
+
+
+def test_roco_mean_std_matches_oracle_convention():
+    from oracle import ref
+    from triton_amd import modules
+    g = torch.Generator().manual_seed(0)
+    s1 = torch.rand(2, 3, 10, generator=g) + 0.5; s2 = s1 * 0.3
+    for causal, sq in ((True, 10), (True, 4), (False, 7)):
+        a = modules.roco_mean_std(s1, s2, sq, causal); b = ref.roco_mean_std(s1, s2, sq, causal)
+        assert torch.allclose(a[0], b[0]) and torch.allclose(a[1], b[1])
+
+
+def test_bench_refuses_more_than_one_gpu():
+    r = subprocess.run(["python", os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "one GPU" in r.stderr
+
+
+def test_flop_and_byte_conventions():
+    from triton_amd import configs
+    assert configs.attn_flops(1, 32, 4096, 4096, 128, True) == 137438953472
+    assert configs.rmsnorm_bytes(4096, 4096) == 67117056
+    assert configs.qkv_gemm_flops(2048, 4096, 4096, 1024) == 103079215104
+    assert configs.attn_flops(1, 71, 2048, 2048, 64, True) == 38117834752
