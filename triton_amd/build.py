@@ -47,7 +47,7 @@ def build(verbose: bool = True, jobs: int = 6) -> str:
     srcs = sources()
     with cf.ThreadPoolExecutor(max_workers=min(jobs, len(srcs))) as ex:
         objs = list(ex.map(_compile, srcs))
-    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB_PATH]
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,--no-undefined", *objs, "-o", LIB_PATH]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stdout}\n{r.stderr}")
