@@ -18,8 +18,11 @@
 // workgroup ids map to different KV heads so that the query heads sharing a KV head land on the same XCD
 // (ids are dealt round-robin to the 8 XCDs) and hit its L2.
 #include "common.h"
+#include <type_traits>
 
 namespace trn {
+
+constexpr int BM = 128;   // queries per workgroup: 4 waves x 32
 
 struct AttnArgs {
     const half_t* q; const half_t* k; const half_t* v; half_t* o;
@@ -32,7 +35,6 @@ struct AttnArgs {
     int causal, q_norm;
 };
 
-constexpr int BM = 128;
 
 
 // XOR swizzle of the 16-byte chunk index within a tile row, as a function of the row.  Tiles are stored
@@ -45,36 +47,40 @@ template <int D> __device__ __forceinline__ int swz(int r) {
     else return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);                        // 8 chunks per 128-byte row
 }
 
-// One wave's share of a K tile and a V tile: NI wave-wide 1 KB loads each, global -> LDS without passing
-// through registers.  Lane i's 16 bytes land at dst + 1024*n + 16*i; which global chunk it fetches (kvo/vvo)
-// decides the swizzle.  soffset = tile offset in bytes (wave-uniform).
+// One wave's share of a K or V stage: NI wave-wide 1 KB loads, global -> LDS without passing through
+// registers.  Load n covers stage rows n*4*RPI + wave*RPI + lane/CPR (RPI rows of CPR 16-byte chunks); lane i's
+// 16 bytes land at the LDS address of that row group + 16*i.  Which global chunk a lane fetches (vo) decides
+// the swizzle; because the row groups of successive loads are a multiple of 16 rows apart the swizzle is the
+// same for all of them, so ONE per-lane offset serves every load and the rest is wave-uniform (soffset).
 #if defined(__HIP_DEVICE_COMPILE__)
-template <int NI>
-__device__ __forceinline__ void fetch_tile(__amdgpu_buffer_rsrc_t krs, __amdgpu_buffer_rsrc_t vrs, half_t* kdst,
-                                           half_t* vdst, const int (&kvo)[NI], const int (&vvo)[NI], int ksoff,
-                                           int vsoff) {
+template <int NI, int D>
+__device__ __forceinline__ void fetch_tile(__amdgpu_buffer_rsrc_t rs, half_t* dst_wave, int vo, int soff, int row_step_bytes) {
+    constexpr int RPI = 64 / (D / 8);
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(krs, (__attribute__((address_space(3))) void*)(kdst + i * 512), 16,
-                                                 kvo[i], ksoff, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(vrs, (__attribute__((address_space(3))) void*)(vdst + i * 512), 16,
-                                                 vvo[i], vsoff, 0, 0);
-    }
+    for (int n = 0; n < NI; ++n)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst_wave + n * 4 * RPI * D),
+                                                 16, vo, soff + n * 4 * row_step_bytes, 0, 0);
 }
 #endif
 
-template <int D, int BN, bool NOISE>
+template <int D, bool NOISE>
 __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-descriptor types and LDS-load builtins exist in the device pass only;
                                       // the host pass needs just the launch stub
-    constexpr int NKS = D / 16;  // MFMA k-steps over head_dim
-    constexpr int NKB = BN / 32; // 32-key blocks per tile
+    constexpr int BN = 64;       // keys per LDS stage (two 32-key blocks)
+    constexpr int NS = D / 16;   // MFMA slots per phase: k-steps of S^T = K Q^T, and (2 key halves) x (D/32) of P V
     constexpr int NDB = D / 32;  // 32-wide blocks of head_dim in O^T
+    constexpr int EPI = 16 / NS; // score elements converted per slot
     constexpr int CPR = D / 8;   // 16-byte chunks per row
-    constexpr int RPI = 64 / CPR;            // tile rows covered by one wave-wide 1 KB load
-    constexpr int NI = BN / (RPI * 4);       // such loads per wave per tile (K and V each)
-    __shared__ __attribute__((aligned(1024))) half_t Ks[2][BN * D];   // double-buffered: tile j+1 lands while j is used
-    __shared__ __attribute__((aligned(1024))) half_t Vs[2][BN * D];
+    constexpr int RPI = 64 / CPR;            // stage rows covered by one wave-wide 1 KB load
+    constexpr int NI = BN / (RPI * 4);       // such loads per wave per stage (K and V each)
+    // Two stages each for K and V, as FOUR separate arrays: the compiler orders an LDS read after every
+    // outstanding global->LDS load that may alias it, and only distinct variables are provably disjoint --
+    // with one [2][..] array every LDS read would wait for the prefetch that was just issued.
+    __shared__ __attribute__((aligned(1024))) half_t Ks0[BN * D];
+    __shared__ __attribute__((aligned(1024))) half_t Ks1[BN * D];
+    __shared__ __attribute__((aligned(1024))) half_t Vs0[BN * D];
+    __shared__ __attribute__((aligned(1024))) half_t Vs1[BN * D];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -89,26 +95,26 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
     const int off = a.Skv - a.Sq;                       // causal: query i sees keys <= i + off
     const int q0 = qt * BM;
-    const int qrow = q0 + wave * 32 + c;                // this lane's query
+    const int wq0 = q0 + wave * 32;                     // first query of this wave
+    const int qrow = wq0 + c;                           // this lane's query
     const int qrow_ld = qrow < a.Sq ? qrow : a.Sq - 1;  // clamp loads; stores are predicated
-    const int wave_last_q = min(q0 + wave * 32 + 31, a.Sq - 1);
 
     // ---- Q^T B-operands: lane holds Q[qrow][ks*16 + 8h .. +7]
-    half8_t qB[NKS];
+    half8_t qB[NS];
     {
         const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * h;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) qB[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 16);
+        for (int ks = 0; ks < NS; ++ks) qB[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 16);
         if (a.q_norm) {   // fused per-head RMSNorm of the query row (other half of the row is in lane^32)
             float ss = 0.f;
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks)
+            for (int ks = 0; ks < NS; ++ks)
 #pragma unroll
                 for (int e = 0; e < 8; ++e) { float f = (float)qB[ks][e]; ss += f * f; }
             ss = half_sum(ss);
             const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
 #pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
+            for (int ks = 0; ks < NS; ++ks) {
                 half8_t gq;
                 if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 16 + 8 * h);
 #pragma unroll
@@ -121,11 +127,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         }
     }
 
-    // ---- LDS read offsets (halfs), lane constants.  K operand: row kb*32+c, logical chunk 2ks+h.
-    int koff[NKS];
+    // ---- LDS read offsets (halfs), lane constants.  K operand: row c of a 32-key block, logical chunk 2ks+h.
+    int koff[NS];
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) koff[ks] = c * D + (((2 * ks + h) ^ swz<D>(c)) << 3);
-    // V^T operand through the transposing read: in each 16-lane group lanes 4r..4r+3 supply tile row r
+    for (int ks = 0; ks < NS; ++ks) koff[ks] = c * D + (((2 * ks + h) ^ swz<D>(c)) << 3);
+    // V^T operand through the transposing read: in each 16-lane group lanes 4r..4r+3 supply stage row r
     // (4 consecutive 8-byte pieces); this lane's piece is row 4h + (lane%16)/4 [+8], head_dim columns
     // db*32 + 16*((lane/16)%2) + 4*(lane%4).
     int voff_lo[NDB], voff_hi[NDB];
@@ -152,155 +158,208 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 
     const float* nrow = NOISE ? a.noise + b * a.nb + head * a.nh + (int64_t)qrow_ld * a.ns : nullptr;
 
-    // ---- staging: direct global -> LDS loads, one tile ahead.  Buffer descriptors give zero fill for
-    // keys past the end (an all-zero V row times P = 0 contributes nothing; garbage could be NaN).
+    // ---- staging: direct global -> LDS loads.  Buffer descriptors give zero fill for keys past the end
+    // (an all-zero V row times P = 0 contributes nothing; garbage could be NaN).
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.k + b * a.kb + kvh * a.kh), 0, (int)(((int64_t)(a.Skv - 1) * a.ks + D) * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.v + b * a.vb + kvh * a.vh), 0, (int)(((int64_t)(a.Skv - 1) * a.vs + D) * 2), 0x00020000);
-    int kvo[NI], vvo[NI];       // per-lane byte offsets of this lane's 16-byte chunk within a tile
-#pragma unroll
-    for (int i = 0; i < NI; ++i) {
-        const int row = (wave * NI + i) * RPI + lane / CPR;
-        const int chunk = (lane % CPR) ^ swz<D>(row);        // LDS slot lane%CPR of that row holds this logical chunk
-        kvo[i] = (int)(row * a.ks * 2) + chunk * 16;
-        vvo[i] = (int)(row * a.vs * 2) + chunk * 16;
-    }
+    const int st_row = wave * RPI + lane / CPR;                      // this lane's row within each 4*RPI-row group
+    const int st_chunk = (lane % CPR) ^ swz<D>(st_row);             // LDS slot lane%CPR of that row holds this logical chunk
+    const int kvo = (int)(st_row * a.ks * 2) + st_chunk * 16;       // per-lane byte offsets within a stage
+    const int vvo = (int)(st_row * a.vs * 2) + st_chunk * 16;
+    const int krow_bytes = (int)(RPI * a.ks * 2), vrow_bytes = (int)(RPI * a.vs * 2);
     const int ktile_bytes = (int)(BN * a.ks * 2), vtile_bytes = (int)(BN * a.vs * 2);
-    // (a __device__ function, not a lambda: with the LDS-load builtin inside a lambda in this kernel template
-    // the host pass silently drops the kernel's launch stub)
-#define TRN_FETCH(jt_, buf_) fetch_tile<NI>(krs, vrs, &Ks[buf_][wave * NI * 512], &Vs[buf_][wave * NI * 512], kvo, vvo, \
-                                           (jt_) * ktile_bytes, (jt_) * vtile_bytes)
-    TRN_FETCH(0, 0);
-    __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0): this wave's loads have landed in LDS
-    __syncthreads();
+#define TRN_FETCH_K(jt_, dst_) fetch_tile<NI, D>(krs, &dst_[wave * RPI * D], kvo, (jt_) * ktile_bytes, krow_bytes)
+#define TRN_FETCH_V(jt_, dst_) fetch_tile<NI, D>(vrs, &dst_[wave * RPI * D], vvo, (jt_) * vtile_bytes, vrow_bytes)
 
-    for (int jt = 0; jt < ntiles; ++jt) {
-        const int kv0 = jt * BN, cur = jt & 1;
-        if (jt + 1 < ntiles) TRN_FETCH(jt + 1, cur ^ 1);   // lands during this tile's MFMAs; last readers of that
-                                                       // buffer passed the barrier that ended the previous tile
+    const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int wb = wq0 + off;          // key index bound of this wave's first query
+    auto needs_mask = [&](int key0) { return (key0 + 32 > a.Skv) || (a.causal && key0 + 31 > wb); };
 
-        // whole tile masked for this wave (wave-uniform)?  It still stages and meets the barrier.
-        if (!(a.causal && kv0 > wave_last_q + off)) {
-            const half_t* Kc = Ks[cur];
-            const half_t* Vc = Vs[cur];
-            // ---- S^T = K Q^T ----
-            float16_t sacc[NKB];
+    // Scores of a 32-key block starting at key0, just produced: (KeyFormer) fold them into the perturbed
+    // row normaliser; mask; block max against the LAZY reference max m.  m is only raised when some row's
+    // true running max exceeds it by more than 2^8: probabilities are then at most 256 (exact in fp16's
+    // range, fp32 sums), O and l stay relative to the same m so the final O/l and m + log2(l) are unchanged,
+    // and the 16*NDB-multiply rescale of O^T runs on the first block or two only instead of on most blocks.
+    // Returns whether a rescale is due (wave-uniform) and the candidate max.
+    auto reduce_block = [&](auto masked_tag, float16_t& sx, int key0, float& smax) __attribute__((always_inline)) {
+        constexpr bool MASKED = decltype(masked_tag)::value;
+        if constexpr (NOISE) {
+            float zmax = m2;
+            float16_t z;
 #pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) {
-                const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int k0 = key0 + 8 * r4 + 4 * h;
+                float4_t gv = {0.f, 0.f, 0.f, 0.f};
+                if constexpr (MASKED) {
+                    const bool any_visible = k0 < a.Skv && (!a.causal || k0 <= qrow + off);
+                    if (any_visible) {
+                        if (k0 + 3 < a.Skv) gv = *reinterpret_cast<const float4_t*>(nrow + k0);
+                        else {
 #pragma unroll
-                for (int ks = 0; ks < NKS; ++ks) {
-                    half8_t ka = *reinterpret_cast<const half8_t*>(&Kc[kb * 32 * D + koff[ks]]);
-                    sacc[kb] = mfma32(ka, qB[ks], ks == 0 ? zero : sacc[kb]);
-                }
-            }
-
-            // ---- perturbed-score row normaliser (KeyFormer): z2 = s*c2 + g*c3, online (m2, l2) ----
-            if constexpr (NOISE) {
-                float zmax = m2;
-                float16_t z[NKB];
-#pragma unroll
-                for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                    for (int r4 = 0; r4 < 4; ++r4) {
-                        const int key0 = kv0 + kb * 32 + 8 * r4 + 4 * h;
-                        float4_t gv = {0.f, 0.f, 0.f, 0.f};
-                        const bool any_visible = key0 < a.Skv && (!a.causal || key0 <= qrow + off);
-                        if (any_visible) {
-                            if (key0 + 3 < a.Skv) gv = *reinterpret_cast<const float4_t*>(nrow + key0);
-                            else {
-#pragma unroll
-                                for (int e = 0; e < 4; ++e) if (key0 + e < a.Skv) gv[e] = nrow[key0 + e];
-                            }
-                        }
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int key = key0 + e;
-                            const bool ok = key < a.Skv && (!a.causal || key <= qrow + off);
-                            float zz = sacc[kb][r4 * 4 + e] * a.c2 + gv[e] * a.c3;
-                            zz = ok ? zz : -INFINITY;
-                            z[kb][r4 * 4 + e] = zz;
-                            zmax = fmaxf(zmax, zz);
+                            for (int e = 0; e < 4; ++e) if (k0 + e < a.Skv) gv[e] = nrow[k0 + e];
                         }
                     }
-                zmax = half_max(zmax);
+                } else {
+                    gv = *reinterpret_cast<const float4_t*>(nrow + k0);
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float zz = sx[r4 * 4 + e] * a.c2 + gv[e] * a.c3;
+                    if constexpr (MASKED) {
+                        const int key = k0 + e;
+                        const bool ok = key < a.Skv && (!a.causal || key <= qrow + off);
+                        zz = ok ? zz : -INFINITY;
+                    }
+                    z[r4 * 4 + e] = zz;
+                    zmax = fmaxf(zmax, zz);
+                }
+            }
+            zmax = half_max(zmax);
+            if (zmax > -INFINITY) {          // a block can be entirely masked for this row pair
                 float sum = 0.f;
 #pragma unroll
-                for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) sum += fast_exp2(z[kb][r] - zmax);
+                for (int r = 0; r < 16; ++r) sum += fast_exp2(z[r] - zmax);
                 l2 = l2 * fast_exp2(m2 - zmax) + sum;
                 m2 = zmax;
             }
-
-            // ---- mask (diagonal / ragged tiles only) ----
-            const bool need_mask = (kv0 + BN > a.Skv) || (a.causal && kv0 + BN - 1 > q0 + wave * 32 + off);
-            if (need_mask) {
+        }
+        if constexpr (MASKED) {
 #pragma unroll
-                for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        const int key = kv0 + kb * 32 + 8 * (r / 4) + 4 * h + (r % 4);
-                        const bool ok = key < a.Skv && (!a.causal || key <= qrow + off);
-                        sacc[kb][r] = ok ? sacc[kb][r] : -INFINITY;
-                    }
-            }
-
-            // ---- online softmax (log2 domain) against a LAZY reference max ----
-            // m is only raised when some row's true running max exceeds it by more than 2^8: probabilities
-            // are then at most 256 (exact in fp16's range, fp32 sums), O and l stay relative to the same m so
-            // the final O/l and m + log2(l) are unchanged, and the 16*NDB-multiply rescale of O^T -- a large
-            // share of the VALU work -- runs on the first tile or two only instead of on most tiles.
-            float smax = -INFINITY;
-#pragma unroll
-            for (int kb = 0; kb < NKB; ++kb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) smax = fmaxf(smax, sacc[kb][r]);
-            smax = half_max(smax) * a.c1;
-            if (__builtin_amdgcn_ballot_w64(smax > m + 8.0f) != 0) {      // wave-uniform
-                const float mnew = fmaxf(m, smax);
-                const float alpha = fast_exp2(m - mnew);
-                l *= alpha;
-#pragma unroll
-                for (int i = 0; i < NDB; ++i)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-                m = mnew;
-            }
-
-            // ---- P^T (fp16) straight into B-operands, O^T += V^T P^T ----
-            // The row sum is taken over the fp16-rounded P (v_dot2_f32_f16 against ones, fp32 accumulate),
-            // i.e. over exactly the values that multiply V.
-            const half2_t ones = {(half_t)1.f, (half_t)1.f};
-#pragma unroll
-            for (int kb = 0; kb < NKB; ++kb) {
-#pragma unroll
-                for (int sp = 0; sp < 2; ++sp) {
-                    half8_t pB;
-#pragma unroll
-                    for (int t = 0; t < 8; t += 2) {
-                        const float p0 = fast_exp2(__builtin_fmaf(sacc[kb][8 * sp + t], a.c1, -m));
-                        const float p1 = fast_exp2(__builtin_fmaf(sacc[kb][8 * sp + t + 1], a.c1, -m));
-                        const half2_t pp = {(half_t)p0, (half_t)p1};
-                        l = __builtin_amdgcn_fdot2(pp, ones, l, false);
-                        pB[t] = pp[0]; pB[t + 1] = pp[1];
-                    }
-#pragma unroll
-                    for (int db = 0; db < NDB; ++db) {
-                        const half_t* vp = &Vc[(kb * 32 + 16 * sp) * D];
-                        half4_t lo = lds_read_tr16(vp + voff_lo[db]);   // keys +0..3 of this lane half, dim db*32+c
-                        half4_t hi = lds_read_tr16(vp + voff_hi[db]);   // keys +8..11
-                        half8_t va = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
-                        oacc[db] = mfma32(va, pB, oacc[db]);
-                    }
-                }
+            for (int r = 0; r < 16; ++r) {
+                const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                const bool ok = key < a.Skv && (!a.causal || key <= qrow + off);
+                sx[r] = ok ? sx[r] : -INFINITY;      // (a select: stale-LDS garbage past the last block never propagates)
             }
         }
+        smax = sx[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) smax = fmaxf(smax, sx[r]);
+        smax = half_max(smax) * a.c1;
+        return __builtin_amdgcn_ballot_w64(smax > m + 8.0f) != 0;
+    };
+    auto rescale = [&](float smax) __attribute__((always_inline)) {
+        const float mnew = fmaxf(m, smax);
+        const float alpha = fast_exp2(m - mnew);
+        l *= alpha;
+#pragma unroll
+        for (int i = 0; i < NDB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        m = mnew;
+    };
 
-        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's share of the next tile is in LDS
-        __syncthreads();                      // next tile visible; this tile's buffer may be overwritten next time
+#ifndef TRN_OPERAND_WINDOW
+#define TRN_OPERAND_WINDOW 2
+#endif
+    constexpr int NQ = TRN_OPERAND_WINDOW < NS ? TRN_OPERAND_WINDOW : NS / 2;   // operand look-ahead in MFMA slots
+    half8_t ka[NQ];    // K operands of the next block's S^T: a rolling window NQ MFMA slots ahead of use
+    half8_t va[NQ];    // V^T operands of this block's P V: likewise
+
+    // One pipeline step for block B whose scores sc are complete, masked and reflected in m:
+    //   phase A: MFMA: S^T of block B+1                  | VALU: P = exp2(sc*c1 - m), fp16, row sum
+    //   phase B: MFMA: O^T += V^T P^T                    | VALU: mask + max of block B+1's scores
+    // A wave issues in order and an MFMA holds the matrix pipe for 8 passes, so program order IS the
+    // schedule: one MFMA, its share of the VALU work and one LDS operand request per slot, with
+    // sched_barrier to keep the compiler from regrouping.  Each operand is requested NQ slots before its
+    // MFMA, into the register its predecessor just vacated:
+    //   phase A slot i < NS-NQ : K operand i+NQ of block B+1 (K1)   later slots : V^T operand i+NQ-NS of block B
+    //   phase B slot i < NS-NQ : V^T operand i+NQ of block B        later slots : K operand i+NQ-NS of block B+2 (K2)
+    // With SYNC (first block of a 64-key tile) the tile hand-over sits NQ slots before the end of phase A: by
+    // then every wave has made its last read of the tile's own K stage (block B+1's last operands) and of the
+    // previous tile's V stage, so after the barrier those two stages are refilled (K two tiles ahead, V one
+    // tile ahead) and all later LDS reads of this and the next step go to the stages that just became visible.
+    auto step = [&](auto masked_tag, auto sync_tag, float16_t& sc, float16_t& sn, const half_t* Vblk, const half_t* K1,
+                    const half_t* K2, int key0_next, auto&& handover) __attribute__((always_inline)) {
+        constexpr bool SYNC = decltype(sync_tag)::value;
+        // The row sum is taken over the fp16-rounded P (v_dot2_f32_f16 against ones, fp32 accumulate),
+        // i.e. over exactly the values that multiply V.
+        const half2_t ones = {(half_t)1.f, (half_t)1.f};
+        half8_t pB[2];
+        auto load_v = [&](int op, int reg) __attribute__((always_inline)) {
+            const half_t* vp = Vblk + 16 * (op / NDB) * D;
+            half4_t lo = lds_read_tr16(vp + voff_lo[op % NDB]);   // keys +0..3 of this lane half, dim db*32+c
+            half4_t hi = lds_read_tr16(vp + voff_hi[op % NDB]);   // keys +8..11
+            va[reg] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+        };
+        // ---- phase A ----
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            if constexpr (SYNC) {
+                if (i == NS - NQ) handover();
+            }
+            sn = mfma32(ka[i % NQ], qB[i], i == 0 ? zero : sn);
+            if (i + NQ < NS) ka[i % NQ] = *reinterpret_cast<const half8_t*>(&K1[koff[i + NQ]]);
+            else load_v(i + NQ - NS, i % NQ);
+#pragma unroll
+            for (int e = 0; e < EPI; e += 2) {
+                const int r = i * EPI + e;
+                const float p0 = fast_exp2(__builtin_fmaf(sc[r], a.c1, -m));
+                const float p1 = fast_exp2(__builtin_fmaf(sc[r + 1], a.c1, -m));
+                const half2_t pp = {(half_t)p0, (half_t)p1};
+                l = __builtin_amdgcn_fdot2(pp, ones, l, false);
+                pB[r / 8][r % 8] = pp[0]; pB[r / 8][r % 8 + 1] = pp[1];
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // ---- phase B ----
+        float smax = 0.f;
+        bool due = false;
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            oacc[i % NDB] = mfma32(va[i % NQ], pB[i / NDB], oacc[i % NDB]);
+            if (i + NQ < NS) load_v(i + NQ, i % NQ);
+            else ka[i % NQ] = *reinterpret_cast<const half8_t*>(&K2[koff[i + NQ - NS]]);
+            if (i == NS / 2) due = reduce_block(masked_tag, sn, key0_next, smax);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (due) rescale(smax);
+    };
+
+    // ---- prologue: K stages 0 and 1 and V stage 0; scores of block 0; first K operands of block 1 ----
+    TRN_FETCH_K(0, Ks0);
+    TRN_FETCH_V(0, Vs0);
+    if (ntiles > 1) TRN_FETCH_K(1, Ks1);
+    __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0): this wave's loads have landed in LDS
+    __syncthreads();
+
+    float16_t sA, sB;                       // scores of the current / next 32-key block (ping-pong)
+    {
+        half8_t k0[NS];
+#pragma unroll
+        for (int i = 0; i < NS; ++i) k0[i] = *reinterpret_cast<const half8_t*>(&Ks0[koff[i]]);
+#pragma unroll
+        for (int i = 0; i < NS; ++i) sA = mfma32(k0[i], qB[i], i == 0 ? zero : sA);
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) ka[i] = *reinterpret_cast<const half8_t*>(&Ks0[32 * D + koff[i]]);
+        float smax;
+        if (reduce_block(std::true_type{}, sA, 0, smax)) rescale(smax);
     }
+
+    // One 64-key tile jt.  Kc = its own K stage (block 1 still has operands to give), Kn = the next tile's
+    // K stage, Vc = its V stage, Vn = the other V stage.
+    auto tile = [&](int jt, half_t* Kc, const half_t* Kn, const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
+        const int kv0 = jt * BN;
+        auto handover = [&]() __attribute__((always_inline)) {
+            __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's share of stages Kn and Vc is in LDS
+            __syncthreads();                      // ... and everyone's; Kc and Vn have had their last readers
+            if (jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
+            if (jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
+        };
+        auto none = [&]() __attribute__((always_inline)) {};
+        // (Past the last tile a K stage holds stale rows; scores computed from them are masked away.)
+        if (needs_mask(kv0 + 32)) step(std::true_type{}, std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
+        else step(std::false_type{}, std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
+        if (needs_mask(kv0 + 64)) step(std::true_type{}, std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
+        else step(std::false_type{}, std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
+    };
+    for (int jt = 0; jt < ntiles; jt += 2) {
+        tile(jt, Ks0, Ks1, Vs0, Vs1);
+        if (jt + 1 < ntiles) tile(jt + 1, Ks1, Ks0, Vs1, Vs0);
+    }
+#undef TRN_FETCH_K
+#undef TRN_FETCH_V
 
     // ---- epilogue: normalise, store O[qrow][d..d+3], LSEs ----
     l = half_sum(l);
@@ -326,12 +385,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #endif
 }
 
-#undef TRN_FETCH
-
-template <int D, int BN, bool NOISE>
-static hipError_t launch_fwd(const AttnArgs& a, hipStream_t s) {
-    const unsigned grid = (unsigned)a.n_qtiles * a.B * a.Hq;
-    hipLaunchKernelGGL((attn_fwd_kernel<D, BN, NOISE>), dim3(grid), dim3(256), 0, s, a);
+template <int D, bool NOISE>
+static hipError_t launch_fwd(AttnArgs a, hipStream_t s) {
+    a.n_qtiles = (a.Sq + BM - 1) / BM;
+    const int64_t grid = (int64_t)a.n_qtiles * a.B * a.Hq;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    hipLaunchKernelGGL((attn_fwd_kernel<D, NOISE>), dim3((unsigned)grid), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
@@ -377,7 +436,7 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     a.q = (const half_t*)q; a.k = (const half_t*)k; a.v = (const half_t*)v; a.o = (half_t*)o;
     a.lse = lse; a.gamma_q = (const half_t*)gamma_q; a.noise = noise; a.lse_pert = lse_pert;
     a.B = d->batch; a.Hq = d->n_q_heads; a.Hkv = d->n_kv_heads; a.Sq = d->seq_q; a.Skv = d->seq_kv;
-    a.n_qtiles = (d->seq_q + BM - 1) / BM;
+    a.n_qtiles = 0;   // set per tile shape at launch
     a.qb = d->q_stride_b; a.qh = d->q_stride_h; a.qs = d->q_stride_s;
     a.kb = d->k_stride_b; a.kh = d->k_stride_h; a.ks = d->k_stride_s;
     a.vb = d->v_stride_b; a.vh = d->v_stride_h; a.vs = d->v_stride_s;
@@ -387,13 +446,12 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
-    if ((int64_t)a.n_qtiles * a.B * a.Hq > 0x7fffffffLL) return TRN_E_SHAPE;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     if (((int64_t)d->seq_kv + 128) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 128) * d->v_stride_s * 2 > 0x7fffffffLL)
         return TRN_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    if (d->head_dim == 128) e = noise ? launch_fwd<128, 64, true>(a, s) : launch_fwd<128, 64, false>(a, s);
-    else e = noise ? launch_fwd<64, 64, true>(a, s) : launch_fwd<64, 64, false>(a, s);
+    if (d->head_dim == 128) e = noise ? launch_fwd<128, true>(a, s) : launch_fwd<128, false>(a, s);
+    else e = noise ? launch_fwd<64, true>(a, s) : launch_fwd<64, false>(a, s);
     return e == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }

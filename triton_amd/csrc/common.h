@@ -26,11 +26,16 @@ __device__ __forceinline__ float16_t mfma32(half8_t a, half8_t b, float16_t c) {
 }
 
 // Combine a value with the one held by the lane 32 away (the other half of a 32x32 accumulator
-// column).  ds_bpermute-based exchange; used once per KV tile, so its cost is noise.
-// (v_permlane32_swap with both operands equal is folded by the compiler as if its two results were
-// the same value, which they are not -- do not use it for this.)
-__device__ __forceinline__ float half_max(float x) { return fmaxf(x, __shfl_xor(x, 32, 64)); }
-__device__ __forceinline__ float half_sum(float x) { return x + __shfl_xor(x, 32, 64); }
+// column).  v_permlane32_swap exchanges the upper half of one register with the lower half of another:
+// starting from two copies of x it leaves {own, other} in the pair (order depends on the lane half), and
+// max / + are commutative.  One VALU op, no LDS traffic -- it must not queue behind the LDS operand
+// prefetches.  Issued as inline asm: the compiler's builtin for this instruction mis-folds its second
+// result when both results feed one operation.  The s_nop covers the VALU-write -> permlane-read hazard.
+__device__ __forceinline__ void swap_halves(float& a, float& b) {
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+__device__ __forceinline__ float half_max(float x) { float a = x, b = x; swap_halves(a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float half_sum(float x) { float a = x, b = x; swap_halves(a, b); return a + b; }
 
 // Transposing LDS read (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane a points at 4 fp16
 // (8 bytes); lanes 4r..4r+3 together supply "row" r = 16 consecutive elements (their addresses need
