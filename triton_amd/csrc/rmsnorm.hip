@@ -13,11 +13,14 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
     int64_t x_outer, int64_t ldx, int64_t y_outer, int64_t ldy, int64_t row_start, float eps) {
     constexpr int ROWS_PER_BLOCK = 256 / LPR;
     const int sub = threadIdx.x % LPR;
-    const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LPR;
-    if (row >= n_rows) return;                       // whole LPR-lane groups leave together
-    const int64_t outer = row / inner_rows, inner = row % inner_rows + row_start;
-    const half_t* xr = x + outer * x_outer + inner * ldx;
-    half_t* yr = y + outer * y_outer + inner * ldy;
+    const uint32_t row = blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / LPR;
+    if (row >= (uint32_t)n_rows) return;             // whole LPR-lane groups leave together
+    // 32-bit row arithmetic: the address must be ready before the first load can issue, and a 64-bit
+    // division on that path costs more than the whole streaming loop of a short row
+    uint32_t outer = 0, inner = row;
+    if (inner_rows != n_rows) { outer = row / (uint32_t)inner_rows; inner = row - outer * (uint32_t)inner_rows; }
+    const half_t* xr = x + (int64_t)outer * x_outer + ((int64_t)inner + row_start) * ldx;
+    half_t* yr = y + (int64_t)outer * y_outer + ((int64_t)inner + row_start) * ldy;
 
     half8_t v[NV];
     float ss = 0.f;
@@ -25,7 +28,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
     for (int i = 0; i < NV; ++i) {
         const int c = (i * LPR + sub) * 8;
         if (c < cols) {
-            v[i] = *reinterpret_cast<const half8_t*>(xr + c);
+            v[i] = __builtin_nontemporal_load(reinterpret_cast<const half8_t*>(xr + c));   // streamed once: keep it out of the caches' way
 #pragma unroll
             for (int e = 0; e < 8; ++e) { float f = (float)v[i][e]; ss += f * f; }
         }
