@@ -145,6 +145,14 @@ int trn_prenorm_qkv_f16(const void* x, const void* gamma /* nullable */,
                         int64_t v_stride_h, int64_t v_stride_s,
                         float eps, int32_t norm, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: a plain 16-bytes-per-lane streaming copy of `bytes`
+ * (a multiple of 16) from src to dst.  bench.py and the profiling recipes run it on a buffer of known size so
+ * that HBM byte counters (FETCH_SIZE / WRITE_SIZE) and achieved GB/s of the real kernels can be scaled
+ * against a kernel whose traffic is known exactly.
+ */
+int trn_calibration_copy(const void* src, void* dst, int64_t bytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,3 +25,26 @@ extern "C" int trn_check_device(void) {
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return TRN_E_ARCH;
     return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? TRN_OK : TRN_E_ARCH;
 }
+
+// Plain streaming copy, 16 bytes per lane, non-temporal both ways: the yardstick that HBM counters and
+// achieved bandwidth of the real kernels are calibrated against.
+namespace trn {
+__global__ __launch_bounds__(256) void calibration_copy_kernel(const uint4_t* __restrict__ src, uint4_t* __restrict__ dst,
+                                                               int64_t n16) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
+}
+}  // namespace trn
+
+extern "C" int trn_calibration_copy(const void* src, void* dst, int64_t bytes, void* stream) {
+    using namespace trn;
+    if (bytes < 0 || bytes % 16) return TRN_E_SHAPE;
+    if (bytes == 0) return TRN_OK;
+    if (!src || !dst) return TRN_E_NULL;
+    if (!aligned16(src) || !aligned16(dst)) return TRN_E_ALIGN;
+    const int64_t n16 = bytes / 16, grid = (n16 + 255) / 256;
+    if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
+    hipLaunchKernelGGL(calibration_copy_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream,
+                       (const uint4_t*)src, (uint4_t*)dst, n16);
+    return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+}

@@ -361,11 +361,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #undef TRN_FETCH_K
 #undef TRN_FETCH_V
 
-    // ---- epilogue: normalise, store O[qrow][d..d+3], LSEs ----
+    // ---- epilogue: normalise; transpose this wave's 32 x D tile through LDS so that the stores are whole
+    // 16-byte-per-lane row segments (the accumulator layout would give 8-byte pieces scattered over 32 rows,
+    // i.e. partial-line writes); LSEs ----
     l = half_sum(l);
     const float inv = 1.0f / l;
-    if (qrow < a.Sq) {
-        half_t* op = a.o + b * a.ob + head * a.oh + (int64_t)qrow * a.os;
+    __syncthreads();                                   // every wave is done with the K/V stages
+    {
+        constexpr int OP = D + 4;                      // row pitch in halfs: 8-byte writes of 32 rows spread over all banks
+        half_t* ot = wave == 0 ? Ks0 : wave == 1 ? Ks1 : wave == 2 ? Vs0 : Vs1;   // 32*OP*2 bytes <= one stage
 #pragma unroll
         for (int db = 0; db < NDB; ++db)
 #pragma unroll
@@ -373,10 +377,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                 half4_t ov;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) ov[e] = (half_t)(oacc[db][r4 * 4 + e] * inv);
-                *reinterpret_cast<half4_t*>(op + db * 32 + 8 * r4 + 4 * h) = ov;
+                *reinterpret_cast<half4_t*>(&ot[c * OP + db * 32 + 8 * r4 + 4 * h]) = ov;
             }
-        if (h == 0 && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + qrow] = (m + fast_log2(l)) * kLn2;
+        __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0): this wave's own writes (no other wave reads them)
+        constexpr int LPRW = D / 8;                    // lanes per output row
+        const int orow = lane / LPRW, ocol = (lane % LPRW) * 8;
+        half_t* ob = a.o + b * a.ob + head * a.oh;
+#pragma unroll
+        for (int j = 0; j < 32 / (64 / LPRW); ++j) {
+            const int r = j * (64 / LPRW) + orow;
+            const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol]);
+            const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol + 4]);
+            if (wq0 + r < a.Sq)
+                *reinterpret_cast<uint4_t*>(ob + (int64_t)(wq0 + r) * a.os + ocol) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+        }
     }
+    if (qrow < a.Sq && h == 0 && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + qrow] = (m + fast_log2(l)) * kLn2;
     if constexpr (NOISE) {
         const float l2s = half_sum(l2);
         if (qrow < a.Sq && h == 0)

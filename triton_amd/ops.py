@@ -170,3 +170,12 @@ def prenorm_qkv(x: torch.Tensor, gamma: Optional[torch.Tensor], wq, wk, wv, q_ou
                                  k_out.stride(1), v_out.stride(0), v_out.stride(1), float(eps), int(bool(norm)),
                                  _stream(x))
     _lib.check("trn_prenorm_qkv_f16", st)
+
+
+def calibration_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """dst <- src with the library's plain streaming copy kernel (measurement yardstick)."""
+    _need(src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous(), "expected contiguous GPU tensors")
+    nbytes = src.numel() * src.element_size()
+    _need(nbytes == dst.numel() * dst.element_size() and nbytes % 16 == 0, "sizes must match and be a multiple of 16 bytes")
+    lib = _lib.load()
+    _lib.check("trn_calibration_copy", lib.trn_calibration_copy(_ptr(src), _ptr(dst), nbytes, _stream(src)))
