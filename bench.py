@@ -267,10 +267,12 @@ def main():
     # HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
     # (recipe and scaling in profiles/); null until that file exists.
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "attn_fwd_llama3_s4096_hbm_traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "attn_fwd_llama3_s4096_hbm_traffic.txt")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("hbm_bytes_per_launch")
+            for ln in f:
+                if ln.startswith("hbm_bytes_per_launch:"):
+                    traffic = int(ln.split(":")[1])
     line = {
         "metric": "attn TFLOP/s + % fp16 MFMA peak (Llama3-8B, S=4096); RMSNorm HBM GB/s",
         "value": round(van["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,

@@ -30,20 +30,26 @@ def kernel_stats(con):
 
 
 def counters(con):
+    """Per kernel: counter sums, dispatch ids and summed durations; plus per-(kernel, grid size) sums so that
+    the calibration copy of one particular size can be singled out."""
     agg = collections.defaultdict(lambda: collections.defaultdict(float))
     disp = collections.defaultdict(set)
     dur = collections.defaultdict(float)
+    bygrid = collections.defaultdict(lambda: collections.defaultdict(float))
+    gdisp = collections.defaultdict(set)
     try:
-        cur = con.execute("select kernel_name, dispatch_id, counter_name, value, duration from counters_collection")
+        cur = con.execute("select kernel_name, dispatch_id, counter_name, value, duration, grid_size from counters_collection")
     except sqlite3.Error:
-        return {}, {}, {}
+        return {}, {}, {}, {}, {}
     seen = set()
-    for name, d, cname, val, du in cur:
+    for name, d, cname, val, du, grid in cur:
         agg[name][cname] += val
         disp[name].add(d)
+        bygrid[(name, grid)][cname] += val
+        gdisp[(name, grid)].add(d)
         if (name, d) not in seen:
             seen.add((name, d)); dur[name] += du
-    return agg, disp, dur
+    return agg, disp, dur, bygrid, gdisp
 
 
 def main():
@@ -58,11 +64,13 @@ def main():
         print(f"{'kernel':72s} {'calls':>6s} {'avg_us':>10s} {'total_us':>11s}")
         for name, calls, total, avg in stats:
             print(f"{short(name):72s} {calls:6d} {avg / 1e3:10.2f} {total / 1e3:11.1f}")
-    agg, disp, dur = counters(con)
+    agg, disp, dur, bygrid, gdisp = counters(con)
     calib = {}
-    for name in agg:
-        if "calibration_copy" in name:
-            calib = {c: v / len(disp[name]) for c, v in agg[name].items()}
+    for (name, grid), vals in bygrid.items():       # the copy launched on exactly --calib-bytes (16 bytes per work-item)
+        if "calibration_copy" in name and a.calib_bytes and grid == a.calib_bytes // 16:
+            calib = {c: v / len(gdisp[(name, grid)]) for c, v in vals.items()}
+            print(f"\ncalibration copy of {a.calib_bytes} bytes: " + ", ".join(f"{c}={v:.1f}" for c, v in sorted(calib.items()))
+                  + f"  ({len(gdisp[(name, grid)])} dispatches)")
     for name in agg:
         if a.filter not in name:
             continue
