@@ -183,8 +183,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     // range, fp32 sums), O and l stay relative to the same m so the final O/l and m + log2(l) are unchanged,
     // and the 16*NDB-multiply rescale of O^T runs on the first block or two only instead of on most blocks.
     // Returns whether a rescale is due (wave-uniform) and the candidate max.
-    auto reduce_block = [&](auto masked_tag, float16_t& sx, int key0, float& smax) __attribute__((always_inline)) {
-        constexpr bool MASKED = decltype(masked_tag)::value;
+    auto reduce_block = [&](bool masked, float16_t& sx, int key0, float& smax) __attribute__((always_inline)) {
+        // `masked` is wave-uniform: the branches below touch only this block's 16 score registers, so the
+        // accumulators never meet a control-flow merge.  (Two whole-step variants selected by a branch cost
+        // dozens of accumulator register copies per step and broke the in-place MFMA accumulation chains.)
         if constexpr (NOISE) {
             float zmax = m2;
             float16_t z;
@@ -192,7 +194,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
             for (int r4 = 0; r4 < 4; ++r4) {
                 const int k0 = key0 + 8 * r4 + 4 * h;
                 float4_t gv = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (MASKED) {
+                if (masked) {
                     const bool any_visible = k0 < a.Skv && (!a.causal || k0 <= qrow + off);
                     if (any_visible) {
                         if (k0 + 3 < a.Skv) gv = *reinterpret_cast<const float4_t*>(nrow + k0);
@@ -206,12 +208,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                 }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
+                    const int key = k0 + e;
+                    const bool ok = !masked || (key < a.Skv && (!a.causal || key <= qrow + off));
                     float zz = sx[r4 * 4 + e] * a.c2 + gv[e] * a.c3;
-                    if constexpr (MASKED) {
-                        const int key = k0 + e;
-                        const bool ok = key < a.Skv && (!a.causal || key <= qrow + off);
-                        zz = ok ? zz : -INFINITY;
-                    }
+                    zz = ok ? zz : -INFINITY;
                     z[r4 * 4 + e] = zz;
                     zmax = fmaxf(zmax, zz);
                 }
@@ -225,7 +225,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
                 m2 = zmax;
             }
         }
-        if constexpr (MASKED) {
+        if (masked) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
@@ -270,7 +270,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     // then every wave has made its last read of the tile's own K stage (block B+1's last operands) and of the
     // previous tile's V stage, so after the barrier those two stages are refilled (K two tiles ahead, V one
     // tile ahead) and all later LDS reads of this and the next step go to the stages that just became visible.
-    auto step = [&](auto masked_tag, auto sync_tag, float16_t& sc, float16_t& sn, const half_t* Vblk, const half_t* K1,
+    auto step = [&](bool masked_next, auto sync_tag, float16_t& sc, float16_t& sn, const half_t* Vblk, const half_t* K1,
                     const half_t* K2, int key0_next, auto&& handover) __attribute__((always_inline)) {
         constexpr bool SYNC = decltype(sync_tag)::value;
         // The row sum is taken over the fp16-rounded P (v_dot2_f32_f16 against ones, fp32 accumulate),
@@ -311,7 +311,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
             oacc[i % NDB] = mfma32(va[i % NQ], pB[i / NDB], oacc[i % NDB]);
             if (i + NQ < NS) load_v(i + NQ, i % NQ);
             else ka[i % NQ] = *reinterpret_cast<const half8_t*>(&K2[koff[i + NQ - NS]]);
-            if (i == NS / 2) due = reduce_block(masked_tag, sn, key0_next, smax);
+            if (i == NS / 2) due = reduce_block(masked_next, sn, key0_next, smax);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (due) rescale(smax);
@@ -334,7 +334,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < NQ; ++i) ka[i] = *reinterpret_cast<const half8_t*>(&Ks0[32 * D + koff[i]]);
         float smax;
-        if (reduce_block(std::true_type{}, sA, 0, smax)) rescale(smax);
+        if (reduce_block(true, sA, 0, smax)) rescale(smax);
     }
 
     // One 64-key tile jt.  Kc = its own K stage (block 1 still has operands to give), Kn = the next tile's
@@ -349,10 +349,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
         };
         auto none = [&]() __attribute__((always_inline)) {};
         // (Past the last tile a K stage holds stale rows; scores computed from them are masked away.)
-        if (needs_mask(kv0 + 32)) step(std::true_type{}, std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
-        else step(std::false_type{}, std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
-        if (needs_mask(kv0 + 64)) step(std::true_type{}, std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
-        else step(std::false_type{}, std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
+        step(needs_mask(kv0 + 32), std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
+        step(needs_mask(kv0 + 64), std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
     };
     for (int jt = 0; jt < ntiles; jt += 2) {
         tile(jt, Ks0, Ks1, Vs0, Vs1);
