@@ -38,6 +38,9 @@ CASES = [
     (1, 5, 5, 16, 1040, 64, False),
     (1, 2, 2, 1, 1, 64, True),
     (1, 2, 1, 129, 257, 128, True),
+    (2, 32, 8, 1024, 1024, 128, True),   # enough workgroups for the 8-wave (256-query) tile shape
+    (2, 32, 8, 1000, 1000, 128, False),  # the same, ragged
+    (1, 72, 1, 1100, 1100, 64, True),
 ]
 
 

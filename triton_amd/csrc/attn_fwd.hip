@@ -22,8 +22,6 @@
 
 namespace trn {
 
-constexpr int BM = 128;   // queries per workgroup: 4 waves x 32
-
 struct AttnArgs {
     const half_t* q; const half_t* k; const half_t* v; half_t* o;
     float* lse; const half_t* gamma_q; const float* noise; float* lse_pert;
@@ -48,23 +46,23 @@ template <int D> __device__ __forceinline__ int swz(int r) {
 }
 
 // One wave's share of a K or V stage: NI wave-wide 1 KB loads, global -> LDS without passing through
-// registers.  Load n covers stage rows n*4*RPI + wave*RPI + lane/CPR (RPI rows of CPR 16-byte chunks); lane i's
+// registers.  Load n covers stage rows n*NW*RPI + wave*RPI + lane/CPR (RPI rows of CPR 16-byte chunks); lane i's
 // 16 bytes land at the LDS address of that row group + 16*i.  Which global chunk a lane fetches (vo) decides
 // the swizzle; because the row groups of successive loads are a multiple of 16 rows apart the swizzle is the
 // same for all of them, so ONE per-lane offset serves every load and the rest is wave-uniform (soffset).
 #if defined(__HIP_DEVICE_COMPILE__)
-template <int NI, int D>
+template <int NI, int D, int NW>
 __device__ __forceinline__ void fetch_tile(__amdgpu_buffer_rsrc_t rs, half_t* dst_wave, int vo, int soff, int row_step_bytes) {
     constexpr int RPI = 64 / (D / 8);
 #pragma unroll
     for (int n = 0; n < NI; ++n)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst_wave + n * 4 * RPI * D),
-                                                 16, vo, soff + n * 4 * row_step_bytes, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst_wave + n * NW * RPI * D),
+                                                 16, vo, soff + n * NW * row_step_bytes, 0, 0);
 }
 #endif
 
-template <int D, bool NOISE>
-__global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
+template <int D, int NW, bool NOISE>
+__global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-descriptor types and LDS-load builtins exist in the device pass only;
                                       // the host pass needs just the launch stub
     constexpr int BN = 64;       // keys per LDS stage (two 32-key blocks)
@@ -73,7 +71,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     constexpr int EPI = 16 / NS; // score elements converted per slot
     constexpr int CPR = D / 8;   // 16-byte chunks per row
     constexpr int RPI = 64 / CPR;            // stage rows covered by one wave-wide 1 KB load
-    constexpr int NI = BN / (RPI * 4);       // such loads per wave per stage (K and V each)
+    constexpr int NI = BN / (RPI * NW);      // such loads per wave per stage (K and V each)
+    constexpr int BM = 32 * NW;              // queries per workgroup: NW waves x 32
     // Two stages each for K and V, as FOUR separate arrays: the compiler orders an LDS read after every
     // outstanding global->LDS load that may alias it, and only distinct variables are provably disjoint --
     // with one [2][..] array every LDS read would wait for the prefetch that was just issued.
@@ -170,8 +169,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     const int vvo = (int)(st_row * a.vs * 2) + st_chunk * 16;
     const int krow_bytes = (int)(RPI * a.ks * 2), vrow_bytes = (int)(RPI * a.vs * 2);
     const int ktile_bytes = (int)(BN * a.ks * 2), vtile_bytes = (int)(BN * a.vs * 2);
-#define TRN_FETCH_K(jt_, dst_) fetch_tile<NI, D>(krs, &dst_[wave * RPI * D], kvo, (jt_) * ktile_bytes, krow_bytes)
-#define TRN_FETCH_V(jt_, dst_) fetch_tile<NI, D>(vrs, &dst_[wave * RPI * D], vvo, (jt_) * vtile_bytes, vrow_bytes)
+#define TRN_FETCH_K(jt_, dst_) fetch_tile<NI, D, NW>(krs, &dst_[wave * RPI * D], kvo, (jt_) * ktile_bytes, krow_bytes)
+#define TRN_FETCH_V(jt_, dst_) fetch_tile<NI, D, NW>(vrs, &dst_[wave * RPI * D], vvo, (jt_) * vtile_bytes, vrow_bytes)
 
     const float16_t zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const int wb = wq0 + off;          // key index bound of this wave's first query
@@ -366,28 +365,34 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
     const float inv = 1.0f / l;
     __syncthreads();                                   // every wave is done with the K/V stages
     {
-        constexpr int OP = D + 4;                      // row pitch in halfs: 8-byte writes of 32 rows spread over all banks
-        half_t* ot = wave == 0 ? Ks0 : wave == 1 ? Ks1 : wave == 2 ? Vs0 : Vs1;   // 32*OP*2 bytes <= one stage
-#pragma unroll
-        for (int db = 0; db < NDB; ++db)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                half4_t ov;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) ov[e] = (half_t)(oacc[db][r4 * 4 + e] * inv);
-                *reinterpret_cast<half4_t*>(&ot[c * OP + db * 32 + 8 * r4 + 4 * h]) = ov;
-            }
-        __builtin_amdgcn_s_waitcnt(0xc07f);            // lgkmcnt(0): this wave's own writes (no other wave reads them)
-        constexpr int LPRW = D / 8;                    // lanes per output row
+        // two passes of D/2 columns each, so that NW waves' staging regions fit in the four stage arrays
+        constexpr int DP = D / 2, OP = DP + 4;         // row pitch in halfs: 8-byte writes of 32 rows spread over all banks
+        constexpr int LPRW = DP / 8, RPS = 64 / LPRW;  // lanes per output row segment, rows per store instruction
+        static_assert(32 * OP * 2 <= BN * D * 2 / (NW / 4), "staging region too large");
+        half_t* arr = (wave / (NW / 4)) == 0 ? Ks0 : (wave / (NW / 4)) == 1 ? Ks1 : (wave / (NW / 4)) == 2 ? Vs0 : Vs1;
+        half_t* ot = arr + (wave % (NW / 4)) * (BN * D / (NW / 4));
         const int orow = lane / LPRW, ocol = (lane % LPRW) * 8;
         half_t* ob = a.o + b * a.ob + head * a.oh;
 #pragma unroll
-        for (int j = 0; j < 32 / (64 / LPRW); ++j) {
-            const int r = j * (64 / LPRW) + orow;
-            const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol]);
-            const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol + 4]);
-            if (wq0 + r < a.Sq)
-                *reinterpret_cast<uint4_t*>(ob + (int64_t)(wq0 + r) * a.os + ocol) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+        for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+            for (int dbl = 0; dbl < NDB / 2; ++dbl)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    half4_t ov;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) ov[e] = (half_t)(oacc[pass * (NDB / 2) + dbl][r4 * 4 + e] * inv);
+                    *reinterpret_cast<half4_t*>(&ot[c * OP + dbl * 32 + 8 * r4 + 4 * h]) = ov;
+                }
+            // (LDS operations of one wave execute in order: no wait needed between its own writes and reads)
+#pragma unroll
+            for (int j = 0; j < 32 / RPS; ++j) {
+                const int r = j * RPS + orow;
+                const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol]);
+                const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[r * OP + ocol + 4]);
+                if (wq0 + r < a.Sq)
+                    *reinterpret_cast<uint4_t*>(ob + (int64_t)(wq0 + r) * a.os + pass * DP + ocol) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+            }
         }
     }
     if (qrow < a.Sq && h == 0 && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + qrow] = (m + fast_log2(l)) * kLn2;
@@ -399,12 +404,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_kernel(const AttnArgs a) {
 #endif
 }
 
-template <int D, bool NOISE>
+template <int D, int NW, bool NOISE>
 static hipError_t launch_fwd(AttnArgs a, hipStream_t s) {
-    a.n_qtiles = (a.Sq + BM - 1) / BM;
+    a.n_qtiles = (a.Sq + 32 * NW - 1) / (32 * NW);
     const int64_t grid = (int64_t)a.n_qtiles * a.B * a.Hq;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((attn_fwd_kernel<D, NOISE>), dim3((unsigned)grid), dim3(256), 0, s, a);
+    hipLaunchKernelGGL((attn_fwd_kernel<D, NW, NOISE>), dim3((unsigned)grid), dim3(NW * 64), 0, s, a);
     return hipGetLastError();
 }
 
@@ -465,7 +470,19 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
         return TRN_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
-    if (d->head_dim == 128) e = noise ? launch_fwd<128, true>(a, s) : launch_fwd<128, false>(a, s);
-    else e = noise ? launch_fwd<64, true>(a, s) : launch_fwd<64, false>(a, s);
+    // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
+    // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
+    // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to
+    // n_qtiles x, so at least four rounds are needed to balance.  Otherwise 4 waves x 32 (two workgroups per CU).
+#ifndef TRN_FORCE_NW
+    const int64_t n_wide = (int64_t)((d->seq_q + 255) / 256) * d->batch * d->n_q_heads;
+    const bool wide = n_wide >= (d->causal ? 1024 : 256);
+#else
+    const bool wide = TRN_FORCE_NW == 8;
+#endif
+#define TRN_LAUNCH(D_, NW_) (noise ? launch_fwd<D_, NW_, true>(a, s) : launch_fwd<D_, NW_, false>(a, s))
+    if (d->head_dim == 128) e = wide ? TRN_LAUNCH(128, 8) : TRN_LAUNCH(128, 4);
+    else e = wide ? TRN_LAUNCH(64, 8) : TRN_LAUNCH(64, 4);
+#undef TRN_LAUNCH
     return e == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }
