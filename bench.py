@@ -205,6 +205,28 @@ def bench_variant(name, steps, warmup):
     return out
 
 
+def mfma_ceiling():
+    """TFLOP/s of the MFMA-only yardstick kernel with all-zero and with random fp16 operands."""
+    import torch
+    from triton_amd import ops
+    out = {}
+    sink = torch.empty(512 * 256, dtype=torch.float32, device="cuda")
+    for name, ops_t in (("zero_operands", torch.zeros(32768, dtype=torch.float16, device="cuda")),
+                        ("random_operands", torch.randn(32768, device="cuda").half())):
+        for _ in range(2):
+            ops.calibration_mfma(ops_t, sink, 4000, 512)
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        flops = 0.0
+        for _ in range(5):
+            flops += ops.calibration_mfma(ops_t, sink, 4000, 512)
+        end.record()
+        torch.cuda.synchronize()
+        out[name] = flops / start.elapsed_time(end) / 1e9
+    return out
+
+
 def cpu_baseline(q, k, v, budget_s):
     """The CPU oracle (oracle/ref.py, eager PyTorch fp32 on the host cores) on a bounded sample of the
     headline workload: whole query heads at the full S=4096, head by head, until the time budget is
@@ -286,6 +308,9 @@ def main():
                      "frac": round(van["kernel_tflops"] / peak, 4), "traffic": traffic,
                      "kernel": "trn::attn_fwd_kernel<128, false>", "kernel_ms": round(van["kernel_ms"], 5)},
     }
+    ceil = mfma_ceiling()
+    line["roofline"]["mfma_only_kernel_tflops"] = {k: round(v, 1) for k, v in ceil.items()}
+    line["roofline"]["frac_of_mfma_only_random_operands"] = round(van["kernel_tflops"] / ceil["random_operands"], 4)
     if "rmsnorm" in extra:
         r = extra["rmsnorm"]
         line["rmsnorm"] = {"value": round(r["gbps"], 1), "unit": "GB/s", "frac_of_hbm_peak": round(r["frac"], 4),

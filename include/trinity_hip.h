@@ -153,6 +153,16 @@ int trn_prenorm_qkv_f16(const void* x, const void* gamma /* nullable */,
  */
 int trn_calibration_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: n_workgroups x 256 threads each issue
+ * iters x 8 back-to-back v_mfma_f32_32x32x16_f16 (n_workgroups*4*iters*8*32768 flop in all) on register
+ * operands read once from `operands` (fp16, >= 65536 bytes; its data pattern sets the switching activity)
+ * and write a checksum to `sink` (>= n_workgroups*256 floats).  Run with all-zero and with random operands it
+ * shows the nominal and the power-limited sustained MFMA rate of the board, the latter being the practical
+ * ceiling for MFMA-bound kernels on real data.
+ */
+int trn_calibration_mfma(const void* operands, float* sink, int32_t iters, int32_t n_workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

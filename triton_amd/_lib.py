@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(HERE, "libtrinity_hip.so")
 EXPORTS = (
     "trn_version", "trn_status_name", "trn_check_device", "trn_rmsnorm_f16",
     "trn_attn_fwd_f16", "trn_attn_colstats_f16", "trn_prenorm_qkv_f16", "trn_calibration_copy",
+    "trn_calibration_mfma",
 )
 
 
@@ -74,6 +75,8 @@ def load() -> C.CDLL:
     lib.trn_prenorm_qkv_f16.argtypes = [vp] * 8 + [i64] * 15 + [f32, i32, vp]
     lib.trn_calibration_copy.restype = C.c_int
     lib.trn_calibration_copy.argtypes = [vp, vp, i64, vp]
+    lib.trn_calibration_mfma.restype = C.c_int
+    lib.trn_calibration_mfma.argtypes = [vp, vp, i32, i32, vp]
     _lib = lib
     return lib
 

@@ -179,3 +179,14 @@ def calibration_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     _need(nbytes == dst.numel() * dst.element_size() and nbytes % 16 == 0, "sizes must match and be a multiple of 16 bytes")
     lib = _lib.load()
     _lib.check("trn_calibration_copy", lib.trn_calibration_copy(_ptr(src), _ptr(dst), nbytes, _stream(src)))
+
+
+def calibration_mfma(operands: torch.Tensor, sink: torch.Tensor, iters: int, n_workgroups: int) -> float:
+    """Launch the MFMA-only yardstick kernel; returns the flop count of the launch."""
+    _dev_half(operands, "operands"); _dev_float(sink, "sink")
+    _need(operands.numel() >= 32768 and operands.is_contiguous(), "operands: need >= 32768 contiguous fp16 values")
+    _need(sink.numel() >= n_workgroups * 256, "sink too small")
+    lib = _lib.load()
+    _lib.check("trn_calibration_mfma", lib.trn_calibration_mfma(_ptr(operands), _ptr(sink), int(iters), int(n_workgroups),
+                                                                _stream(operands)))
+    return float(n_workgroups) * 4 * iters * 8 * 32768.0
