@@ -8,11 +8,14 @@
 // row scale to the fp32 accumulator at the end ((x*r)@W == r*(x@W)).
 //
 // MFMA mapping (32x32x16 fp16): the product is formed transposed, C^T[n][t] = W^T[n][k] X^T[k][t], so that a
-// lane ends up with 4 consecutive output columns of ONE token (8-byte stores, one rstd per lane).  W is
-// [hidden][n] row-major with the contraction index running down its rows; the W^T A-operand is fetched from
-// the row-major LDS tile with the transposing read ds_read_b64_tr_b16.  X^T is the B operand (16-byte reads).
-// 256 threads = 4 waves in a 2x2 arrangement, each wave a 64x64 sub-tile; global loads for the next k-tile
-// are issued into registers before the MFMAs of the current one.
+// lane ends up with 4 consecutive output columns of ONE token (one rstd per lane).  W is [hidden][n] row-major
+// with the contraction index running down its rows: its tiles go straight from global memory into LDS
+// (buffer_load ... lds), row-major with an XOR chunk swizzle, and the W^T A-operand is fetched with the
+// transposing LDS read ds_read_b64_tr_b16.  X^T is the B operand (16-byte reads of a padded tile that was
+// written from registers).  256 threads = 4 waves in a 2x2 arrangement, each wave a 64x64 sub-tile.  Both
+// tiles are double-buffered: the W fetch and the X global loads of k-tile j+1 are issued before the MFMAs of
+// k-tile j, one barrier per k-tile.  The epilogue transposes each wave's tile through LDS so that the stores
+// are whole 16-byte-per-lane row segments.
 #include "common.h"
 
 namespace trn {
@@ -22,7 +25,7 @@ struct ProjOut { const half_t* w; half_t* out; int64_t ldw, stride_h, stride_s; 
 struct GemmArgs {
     const half_t* x; const half_t* gamma;
     ProjOut p[3];
-    int T, K, head_dim, n_mtiles;
+    int T, K, head_dim, n_mtiles, n_panels, panels_per_xcd;
     int64_t ldx;
     float eps;
     int norm;
@@ -30,64 +33,106 @@ struct GemmArgs {
 
 constexpr int GBM = 128, GBN = 128, GBK = 64;
 
+// chunk swizzle of a 256-byte LDS row (16 chunks of 16 bytes) as a function of the row: a bit permutation of
+// the row's low 4 bits under which 4 consecutive rows read over 4 consecutive chunks (one phase of the
+// transposing read) touch every bank once
+__device__ __forceinline__ int wswz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
 __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
-    constexpr int XP = GBK + 8;    // X tile pitch (halfs)
-    constexpr int WP = GBN + 8;    // W tile pitch (halfs)
-    __shared__ __attribute__((aligned(16))) half_t Xs[GBM * XP];
-    __shared__ __attribute__((aligned(16))) half_t Ws[GBK * WP];
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
+    constexpr int XP = GBK + 8;    // X tile pitch (halfs): rows 36 banks apart -> conflict-free 16-byte row reads
+    // separate arrays per stage: the compiler orders LDS reads after outstanding global->LDS loads that may
+    // alias them, and only distinct variables are provably disjoint
+    __shared__ __attribute__((aligned(1024))) half_t Ws0[GBK * GBN];
+    __shared__ __attribute__((aligned(1024))) half_t Ws1[GBK * GBN];
+    __shared__ __attribute__((aligned(16))) half_t Xs0[GBM * XP];
+    __shared__ __attribute__((aligned(16))) half_t Xs1[GBM * XP];
     __shared__ float rstd_s[GBM];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm = wave & 1, wn = wave >> 1;
-    const int tr_row = (lane & 15) >> 2, tr_col = ((lane >> 4) & 1) * 16 + (lane & 3) * 4;
 
-    const int mt = blockIdx.x % a.n_mtiles, nt_all = blockIdx.x / a.n_mtiles;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  XCD x owns a contiguous run of
+    // 128-column panels of W and walks the token tiles fastest, so the workgroups resident on it together
+    // share a few W panels and each X slab between them instead of every XCD streaming all of W and X.
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int mt = local % a.n_mtiles, nt_all = xcd * a.panels_per_xcd + local / a.n_mtiles;
+    if (nt_all >= a.n_panels) return;
     const int pi = nt_all >= a.p[2].tile0 ? 2 : (nt_all >= a.p[1].tile0 ? 1 : 0);
     const ProjOut P = a.p[pi];
     const int n0 = (nt_all - P.tile0) * GBN, m0 = mt * GBM;
 
-    // fixed per-thread staging coordinates
-    const int xr = tid >> 3, xc = (tid & 7) * 8;       // X: rows xr + 32*i, 8 halfs at column xc
-    const int wr = tid >> 4, wc = (tid & 15) * 8;      // W: rows wr + 16*i, 8 halfs at column wc
-    uint4_t xreg[4], wreg[4];
-    float ss[4] = {0.f, 0.f, 0.f, 0.f};
+    // ---- W: direct global -> LDS.  One wave-wide load covers 4 rows of 256 bytes; load i of this wave covers
+    // stage rows 16*i + 4*wave + lane/16, so the swizzle (a function of row % 16) is the same for all four
+    // and one per-lane offset serves them.
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)P.w, 0, (int)(((int64_t)(a.K - 1) * P.ldw + P.n) * 2), 0x00020000);
+    const int w_row = 4 * wave + lane / 16;
+    const int w_vo = (int)(w_row * P.ldw * 2) + (n0 + (((lane & 15) ^ wswz(w_row)) << 3)) * 2;
+    const int w_row16 = (int)(16 * P.ldw * 2), w_tile = (int)(GBK * P.ldw * 2);
+#define TRN_FETCH_W(kt_, dst_)                                                                                   \
+    _Pragma("unroll") for (int i_ = 0; i_ < 4; ++i_) __builtin_amdgcn_raw_ptr_buffer_load_lds(                  \
+        wrs, (__attribute__((address_space(3))) void*)(&dst_[(16 * i_ + 4 * wave) * GBN]), 16, w_vo,             \
+        (kt_) * w_tile + i_ * w_row16, 0, 0)
 
-    auto fetch = [&](int k0) {
+    // ---- X: global -> registers (gamma, sum of squares) -> LDS.  Thread covers rows xr + 32*i, 8 halfs at xc.
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)a.x, 0, (int)(((int64_t)(a.T - 1) * a.ldx + a.K) * 2), 0x00020000);
+    const int xr = tid >> 3, xc = (tid & 7) * 8;
+    int x_vo[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int t = m0 + xr + 32 * i, k = k0 + xc;
-            xreg[i] = uint4_t{0u, 0u, 0u, 0u};
-            if (t < a.T && k < a.K) xreg[i] = *reinterpret_cast<const uint4_t*>(a.x + (int64_t)t * a.ldx + k);
-        }
+    for (int i = 0; i < 4; ++i) {
+        const int t = m0 + xr + 32 * i;
+        x_vo[i] = t < a.T ? (int)(t * a.ldx * 2) + xc * 2 : 0x7ffffff0;     // rows past the end: out of range -> zeros
+    }
+    uint4_t xreg[4];
+    half8_t greg = {0, 0, 0, 0, 0, 0, 0, 0};
+    float ss[4] = {0.f, 0.f, 0.f, 0.f};
+    const bool use_g = a.gamma != nullptr && a.norm;
+    const bool ragged_k = (a.K % GBK) != 0;
+    auto fetch_x = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int k = k0 + wr + 16 * i, n = n0 + wc;
-            wreg[i] = uint4_t{0u, 0u, 0u, 0u};
-            if (k < a.K && n < P.n) wreg[i] = *reinterpret_cast<const uint4_t*>(P.w + (int64_t)k * P.ldw + n);
-        }
+        for (int i = 0; i < 4; ++i) xreg[i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, x_vo[i], kt * GBK * 2, 0);
+        if (use_g) greg = kt * GBK + xc < a.K ? *reinterpret_cast<const half8_t*>(a.gamma + kt * GBK + xc) : half8_t{0, 0, 0, 0, 0, 0, 0, 0};
     };
-    auto stash = [&](int k0) {
-        half8_t gv;
-        const bool use_g = a.gamma != nullptr && a.norm;
-        if (use_g) {
-            gv = half8_t{0, 0, 0, 0, 0, 0, 0, 0};
-            if (k0 + xc < a.K) gv = *reinterpret_cast<const half8_t*>(a.gamma + k0 + xc);
-        }
+    // Packed fp16 arithmetic keeps this off the critical path (the MFMAs of a k-tile take 512 cycles per wave):
+    // x*gamma as one fp16 multiply per pair is the correctly rounded product, i.e. what an fp32 multiply rounded
+    // to fp16 gives, and the squares are summed two at a time into fp32 by the dot-product instruction.
+    auto stash_x = [&](int kt, half_t* Xd) __attribute__((always_inline)) {
+        // columns past hidden hold the next row's data: ignore them (only the last k-tile can have any)
+        const bool drop = ragged_k && kt * GBK + xc >= a.K;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             half8_t xv = __builtin_bit_cast(half8_t, xreg[i]);
+            if (ragged_k) { if (drop) xv = half8_t{0, 0, 0, 0, 0, 0, 0, 0}; }
             if (a.norm) {
 #pragma unroll
-                for (int e = 0; e < 8; ++e) { const float f = (float)xv[e]; ss[i] += f * f; }
-                if (use_g) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) xv[e] = (half_t)((float)xv[e] * (float)gv[e]);
+                for (int e = 0; e < 4; ++e) {
+                    const half2_t p = {xv[2 * e], xv[2 * e + 1]};
+                    ss[i] = __builtin_amdgcn_fdot2(p, p, ss[i], false);
                 }
+                if (use_g) xv = xv * greg;
             }
-            *reinterpret_cast<half8_t*>(&Xs[(xr + 32 * i) * XP + xc]) = xv;
-            *reinterpret_cast<uint4_t*>(&Ws[(wr + 16 * i) * WP + wc]) = wreg[i];
+            *reinterpret_cast<half8_t*>(&Xd[(xr + 32 * i) * XP + xc]) = xv;
         }
     };
+
+    // ---- LDS read offsets (halfs).  X^T B-operand: row wm*64 + mb*32 + c, columns ks*16 + 8h.
+    const int xoff = (wm * 64 + c) * XP + 8 * h;
+    // W^T A-operand via the transposing read: lane's piece is stage row ks*16 + 8h + (lane%16)/4 [+4], columns
+    // wn*64 + nb*32 + 16*((lane/16)%2) + 4*(lane%4)
+    int woff_lo[2], woff_hi[2];
+    {
+        const int rl = 8 * h + ((lane & 15) >> 2), rh = rl + 4;
+        const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), sub = (lane & 1) * 4;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            const int chunk = wn * 8 + nb * 4 + lc;
+            woff_lo[nb] = rl * GBN + ((chunk ^ wswz(rl)) << 3) + sub;
+            woff_hi[nb] = rh * GBN + ((chunk ^ wswz(rh)) << 3) + sub;
+        }
+    }
 
     float16_t acc[2][2];   // [n block][m block]
 #pragma unroll
@@ -98,22 +143,25 @@ __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
             for (int r = 0; r < 16; ++r) acc[i][jn][r] = 0.f;
 
     const int nk = (a.K + GBK - 1) / GBK;
-    fetch(0);
-    for (int kt = 0; kt < nk; ++kt) {
-        __syncthreads();               // previous tile's MFMAs have read LDS
-        stash(kt * GBK);
-        __syncthreads();
-        if (kt + 1 < nk) fetch((kt + 1) * GBK);   // in flight during the MFMAs below
+    TRN_FETCH_W(0, Ws0);
+    fetch_x(0);
+    stash_x(0, Xs0);
+    __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0)
+    __syncthreads();
+
+    auto ktile = [&](int kt, const half_t* Wc, const half_t* Xc, half_t* Wn, half_t* Xn) __attribute__((always_inline)) {
+        const bool more = kt + 1 < nk;
+        if (more) { TRN_FETCH_W(kt + 1, Wn); fetch_x(kt + 1); }      // land during the MFMAs below
 #pragma unroll
         for (int ks = 0; ks < GBK / 16; ++ks) {
             half8_t xb[2], wa[2];
 #pragma unroll
             for (int mb = 0; mb < 2; ++mb)
-                xb[mb] = *reinterpret_cast<const half8_t*>(&Xs[(wm * 64 + mb * 32 + c) * XP + ks * 16 + 8 * h]);
+                xb[mb] = *reinterpret_cast<const half8_t*>(&Xc[xoff + mb * 32 * XP + ks * 16]);
 #pragma unroll
             for (int nb = 0; nb < 2; ++nb) {
-                const half_t* wp = &Ws[(ks * 16 + 8 * h + tr_row) * WP + wn * 64 + nb * 32 + tr_col];
-                half4_t lo = lds_read_tr16(wp), hi = lds_read_tr16(wp + 4 * WP);
+                half4_t lo = lds_read_tr16(&Wc[ks * 16 * GBN + woff_lo[nb]]);
+                half4_t hi = lds_read_tr16(&Wc[ks * 16 * GBN + woff_hi[nb]]);
                 wa[nb] = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             }
 #pragma unroll
@@ -121,7 +169,15 @@ __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
 #pragma unroll
                 for (int mb = 0; mb < 2; ++mb) acc[nb][mb] = mfma32(wa[nb], xb[mb], acc[nb][mb]);
         }
+        if (more) stash_x(kt + 1, Xn);            // nobody reads Xn: its last readers passed the previous barrier
+        __builtin_amdgcn_s_waitcnt(0x0f70);       // vmcnt(0): this wave's share of the next W stage is in LDS
+        __syncthreads();
+    };
+    for (int kt = 0; kt < nk; kt += 2) {
+        ktile(kt, Ws0, Xs0, Ws1, Xs1);
+        if (kt + 1 < nk) ktile(kt + 1, Ws1, Xs1, Ws0, Xs0);
     }
+#undef TRN_FETCH_W
 
     // row rstd: the 8 threads that staged a row's chunks hold its partial sums of squares
     if (a.norm) {
@@ -134,24 +190,37 @@ __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
     }
     __syncthreads();
 
+    // ---- epilogue: scale, transpose this wave's 64 x 64 tile through LDS (stage memory is free now), store
+    // 16 bytes per lane: 8 lanes cover the 64 columns of a token, 8 tokens per store instruction
+    {
+        constexpr int OP = 64 + 4;                          // pitch in halfs
+        half_t* ot = (wave == 0 ? Ws0 : wave == 1 ? Ws1 : wave == 2 ? Xs0 : Xs1);   // 64*68*2 = 8704 bytes <= a stage
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb) {
-        const int tl = wm * 64 + mb * 32 + c, t = m0 + tl;
-        if (t >= a.T) continue;
-        const float r = a.norm ? rstd_s[tl] : 1.0f;
+        for (int mb = 0; mb < 2; ++mb) {
+            const float r = a.norm ? rstd_s[wm * 64 + mb * 32 + c] : 1.0f;
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb)
+            for (int nb = 0; nb < 2; ++nb)
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int n = n0 + wn * 64 + nb * 32 + 8 * r4 + 4 * h;
-                if (n >= P.n) continue;
-                half4_t ov;
+                for (int r4 = 0; r4 < 4; ++r4) {
+                    half4_t ov;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) ov[e] = (half_t)(acc[nb][mb][r4 * 4 + e] * r);
-                half_t* dst = P.out + (int64_t)(n / a.head_dim) * P.stride_h + (int64_t)t * P.stride_s + (n % a.head_dim);
-                *reinterpret_cast<half4_t*>(dst) = ov;
-            }
+                    for (int e = 0; e < 4; ++e) ov[e] = (half_t)(acc[nb][mb][r4 * 4 + e] * r);
+                    *reinterpret_cast<half4_t*>(&ot[(mb * 32 + c) * OP + nb * 32 + 8 * r4 + 4 * h]) = ov;
+                }
+        }
+        // (LDS operations of one wave execute in order: its reads below see its writes above)
+        const int orow = lane >> 3, ocol = (lane & 7) * 8;
+        const int n = n0 + wn * 64 + ocol;
+        half_t* obase = P.out + (int64_t)(n / a.head_dim) * P.stride_h + (n % a.head_dim);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int tl = j * 8 + orow, t = m0 + wm * 64 + tl;
+            const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol]);
+            const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol + 4]);
+            if (t < a.T && n < P.n) *reinterpret_cast<uint4_t*>(obase + (int64_t)t * P.stride_s) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+        }
     }
+#endif
 }
 
 }  // namespace trn
@@ -173,10 +242,11 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     const void* ptrs[] = {x, wq, wk, wv, q, k, v};
     for (const void* p : ptrs) if (!aligned16(p)) return TRN_E_ALIGN;
     if (gamma && !aligned16(gamma)) return TRN_E_ALIGN;
-    const int64_t pitches[] = {ldx, ldwq, ldwk, ldwv};
-    for (int64_t p : pitches) if (!pitch16(p, 2)) return TRN_E_ALIGN;
-    const int64_t ostr[] = {q_stride_h, q_stride_s, k_stride_h, k_stride_s, v_stride_h, v_stride_s};
-    for (int64_t p : ostr) if ((p * 2) % 8) return TRN_E_ALIGN;     // 8-byte output stores
+    const int64_t pitches[] = {ldx, ldwq, ldwk, ldwv, q_stride_h, q_stride_s, k_stride_h, k_stride_s, v_stride_h, v_stride_s};
+    for (int64_t p : pitches) if (!pitch16(p, 2)) return TRN_E_ALIGN;     // 16-byte loads and stores
+    // X and W tiles are fetched with 32-bit buffer offsets
+    const int64_t spans[] = {(tokens + GBM) * ldx * 2, (hidden + GBK) * ldwq * 2, (hidden + GBK) * ldwk * 2, (hidden + GBK) * ldwv * 2};
+    for (int64_t sp : spans) if (sp > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
 
     GemmArgs a;
     a.x = (const half_t*)x; a.gamma = (const half_t*)gamma;
@@ -186,7 +256,9 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0};
     a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, tq};
     a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, tq + tkv};
-    const int64_t grid = (int64_t)a.n_mtiles * (tq + 2 * tkv);
+    a.n_panels = tq + 2 * tkv;
+    a.panels_per_xcd = (a.n_panels + 7) / 8;
+    const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
     if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
     hipLaunchKernelGGL(prenorm_qkv_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
