@@ -21,7 +21,10 @@ def weights(g, K, nq, nkv, std=0.02):
 
 @pytest.mark.parametrize("T,K,nq,nkv,D,norm", [(256, 512, 512, 128, 128, True), (130, 520, 192, 64, 64, True),
                                               (16, 4096, 4096, 4096, 128, False), (2048, 4096, 4096, 1024, 128, True),
-                                              (1, 64, 64, 64, 64, True), (16, 4544, 4544, 64, 64, True)])
+                                              (1, 64, 64, 64, 64, True), (16, 4544, 4544, 64, 64, True),
+                                              # 256 x 256 tiling (>= 128 of its tiles): ragged tokens and hidden,
+                                              # a nearly empty K/V panel, no norm
+                                              (1000, 520, 6144, 1024, 128, True), (300, 200, 16384, 64, 64, False)])
 def test_qkv_projection_parity(T, K, nq, nkv, D, norm):
     from triton_amd import ops
     g = torch.Generator().manual_seed(42)
@@ -55,3 +58,33 @@ def test_projection_into_kv_cache_rows():
     q, k, v = ref._decode_qkv(X, *W, D, False)
     assert torch.equal(Kd[:, :P].cpu(), Kc[:, :P]) and torch.equal(Vd[:, :P].cpu(), Vc[:, :P])
     close(Kd[:, P:], k, atol=1e-3); close(Vd[:, P:], v, atol=1e-3); close(Qd, q, atol=1e-3)
+
+
+@pytest.mark.parametrize("T,K,nq,nkv,D", [(200, 136, 256, 64, 64),         # 128 x 128 tiling
+                                         (600, 136, 5120, 512, 128)])      # 256 x 256 tiling
+def test_projection_reads_and_writes_stay_inside_its_views(T, K, nq, nkv, D):
+    """Operands are padded views cut out of NaN-filled buffers, hidden and tokens are ragged: a tile load that strays
+    past a row or the end of a view pulls NaN into the product, a store that strays overwrites the NaN padding."""
+    from triton_amd import ops
+    g = torch.Generator().manual_seed(7)
+    x = ref.randn_half((T, K), g); gamma = ref.randn_half((K,), g, 1.0, 0.02)
+    wq, wk, wv = weights(g, K, nq, nkv)
+    nan = float("nan")
+
+    def padded(t, pad):
+        buf = torch.full((t.shape[0] + 3, t.shape[1] + pad), nan, dtype=torch.float16, device="cuda")
+        buf[1:1 + t.shape[0], :t.shape[1]] = t.cuda()
+        return buf, buf[1:1 + t.shape[0], :t.shape[1]]
+
+    (_, xd), (_, wqd), (_, wkd), (_, wvd) = padded(x, 8), padded(wq, 16), padded(wk, 8), padded(wv, 24)
+    outs = []
+    for n in (nq, nkv, nkv):
+        buf = torch.full((T + 2, n + 8), nan, dtype=torch.float16, device="cuda")
+        outs.append((buf, buf[1:1 + T, :n]))
+    views = [o[1].unflatten(1, (n // D, D)).permute(1, 0, 2) for o, n in zip(outs, (nq, nkv, nkv))]
+    ops.prenorm_qkv(xd, gamma.cuda(), wqd, wkd, wvd, views[0], views[1], views[2], 1e-5, True)
+    torch.cuda.synchronize()
+    want = ref.qkv_project(x[None], gamma, wq, wk, wv, 1e-5, True)
+    for (buf, view), w in zip(outs, want):
+        close(view, w[0])
+        assert torch.isnan(buf[0]).all() and torch.isnan(buf[T + 1]).all() and torch.isnan(buf[:, view.shape[1]:]).all()

@@ -16,27 +16,11 @@
 // tiles are double-buffered: the W fetch and the X global loads of k-tile j+1 are issued before the MFMAs of
 // k-tile j, one barrier per k-tile.  The epilogue transposes each wave's tile through LDS so that the stores
 // are whole 16-byte-per-lane row segments.
-#include "common.h"
+#include "prenorm_qkv.h"
 
 namespace trn {
 
-struct ProjOut { const half_t* w; half_t* out; int64_t ldw, stride_h, stride_s; int n; int tile0; };
-
-struct GemmArgs {
-    const half_t* x; const half_t* gamma;
-    ProjOut p[3];
-    int T, K, head_dim, n_mtiles, n_panels, panels_per_xcd;
-    int64_t ldx;
-    float eps;
-    int norm;
-};
-
 constexpr int GBM = 128, GBN = 128, GBK = 64;
-
-// chunk swizzle of a 256-byte LDS row (16 chunks of 16 bytes) as a function of the row: a bit permutation of
-// the row's low 4 bits under which 4 consecutive rows read over 4 consecutive chunks (one phase of the
-// transposing read) touch every bank once
-__device__ __forceinline__ int wswz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
@@ -251,11 +235,15 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     GemmArgs a;
     a.x = (const half_t*)x; a.gamma = (const half_t*)gamma;
     a.T = (int)tokens; a.K = (int)hidden; a.head_dim = (int)head_dim; a.ldx = ldx; a.eps = eps; a.norm = norm ? 1 : 0;
+    a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0};
+    a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, 0};
+    a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, 0};
+    // 256 x 256 tiles once they alone occupy at least half of the 256 CUs; 128 x 128 tiles below that (decode
+    // and short prefills, where the number of workgroups matters more than the work per staged byte)
+    if (prenorm_qkv_wide_tiles(tokens, n_q, n_kv) >= 128) return launch_prenorm_qkv_wide(a, n_q, n_kv, (hipStream_t)stream);
     a.n_mtiles = (int)((tokens + GBM - 1) / GBM);
     const int tq = (int)((n_q + GBN - 1) / GBN), tkv = (int)((n_kv + GBN - 1) / GBN);
-    a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0};
-    a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, tq};
-    a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, tq + tkv};
+    a.p[1].tile0 = tq; a.p[2].tile0 = tq + tkv;
     a.n_panels = tq + 2 * tkv;
     a.panels_per_xcd = (a.n_panels + 7) / 8;
     const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
