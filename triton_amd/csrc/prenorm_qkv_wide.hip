@@ -9,7 +9,7 @@
 //     register staging and no LDS writes from the VALU.  gamma is multiplied into the X operand after it is read
 //     back from LDS (one packed fp16 multiply per pair: the correctly rounded product), and the waves of the
 //     first column group also sum its squares with the fp32 dot-product instruction for the row rstd.
-//   * Four stages of 32 contraction columns: a stage is requested two and a half k-tiles before its first use,
+//   * Four stages of 32 contraction columns: a stage is requested three k-tiles before its first use,
 //     which at 256 x 256 flops per staged column covers the L2 / HBM latency.
 //   * The one barrier per k-tile sits between the two 16-column halves of the tile's MFMAs, after the second
 //     half's operands are already in registers: waves reach it with MFMAs in flight, and the first operands of
@@ -178,11 +178,12 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     // The k-tile loop runs in whole turns of the 4-stage ring and always fetches ahead: k-tiles past hidden
     // fetch zeros (out-of-range loads) and add nothing, which keeps the loop free of tail branches and the count
     // of loads in flight, on which the waits below rely, the same in every iteration.
-    // ---- prologue: three stages and two gamma slices in flight, then the first operands
-    if (use_g) { fetch_g(0, g0); fetch_g(1, g1); }
+    // ---- prologue: all four stages and three gamma slices in flight, then the first operands
+    if (use_g) { fetch_g(0, g0); fetch_g(1, g1); fetch_g(2, g2); }
     TRN_FETCH(0, Xs0, Ws0);
     TRN_FETCH(1, Xs1, Ws1);
     TRN_FETCH(2, Xs2, Ws2);
+    TRN_FETCH(3, Xs3, Ws3);
     __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0)
     __syncthreads();
 #pragma unroll
@@ -197,30 +198,31 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     }
     xv = xv * g0[0];
 
-    // k-tile kt: stage kt%4 is current, (kt+1)%4 is read from the barrier on, (kt+3)%4 is refilled after it
-    auto ktile = [&](int kt, const half_t* Xc, const half_t* Wc, const half_t* Xn, const half_t* Wn, half_t* Xf,
-                     half_t* Wf, const half8_t (&gc)[2], const half8_t (&gn)[2], half8_t (&gf)[2])
-                        __attribute__((always_inline)) {
+    // k-tile kt reads stage kt%4: the operands of its first step during the second step of k-tile kt-1, those of
+    // its second step during its first.  From the barrier between the two steps on, the stage is free and is
+    // refilled with k-tile kt+4 -- three k-tiles before that one's barrier.
+    auto ktile = [&](int kt, half_t* Xc, half_t* Wc, const half_t* Xn, const half_t* Wn, const half8_t (&gc)[2],
+                     const half8_t (&gn)[2], half8_t (&gf)[2]) __attribute__((always_inline)) {
         step(xv, xb0, wa0, gc[0], xb1, wa1, Xc, Wc, 1, gc[1], [&](int) __attribute__((always_inline)) {});
         // Stage kt+1 must have landed.  Loads complete in issue order, and behind this wave's share of that stage
-        // only the gamma slice of k-tile kt+1 (2 loads) and stage kt+2 (8 loads) have been issued.
-        if (use_g) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f78);
+        // only the refills and gamma slices of the last two k-tiles (2 x (8 + 2) loads) have been issued.
+        // lgkmcnt(0): this wave's reads of stage kt have returned, so the refill cannot overtake them.
+        if (use_g) __builtin_amdgcn_s_waitcnt(0x4074); else __builtin_amdgcn_s_waitcnt(0x4070);
         // A bare barrier: __syncthreads() would first drain every load in flight, the prefetched stages included.
-        // Nothing else needs ordering here -- in this loop LDS is written only by those loads, and the LDS reads of
-        // stage kt-1 returned before the MFMAs that consumed them were issued.
-        __builtin_amdgcn_s_barrier();       // everyone's share landed; nobody still reads stage kt-1
+        // Nothing else needs ordering here -- in this loop LDS is written only by those loads.
+        __builtin_amdgcn_s_barrier();       // everyone's share landed; nobody still reads stage kt
         __builtin_amdgcn_sched_barrier(0);
         step(xv, xb1, wa1, gc[1], xb0, wa0, Xn, Wn, 0, gn[0], [&](int i) __attribute__((always_inline)) {
-            // gamma two tiles ahead and before the stage loads: its use never has to wait for a stage
-            if (i == 0 && use_g) fetch_g(kt + 2, gf);
-            TRN_FETCH_ONE(kt + 3, Xf, Wf, i);
+            // gamma three tiles ahead and before the stage loads: its use never has to wait for a stage
+            if (i == 0 && use_g) fetch_g(kt + 3, gf);
+            TRN_FETCH_ONE(kt + 4, Xc, Wc, i);
         });
     };
     for (int kt = 0; kt < nk; kt += 4) {
-        ktile(kt, Xs0, Ws0, Xs1, Ws1, Xs3, Ws3, g0, g1, g2);
-        ktile(kt + 1, Xs1, Ws1, Xs2, Ws2, Xs0, Ws0, g1, g2, g3);
-        ktile(kt + 2, Xs2, Ws2, Xs3, Ws3, Xs1, Ws1, g2, g3, g0);
-        ktile(kt + 3, Xs3, Ws3, Xs0, Ws0, Xs2, Ws2, g3, g0, g1);
+        ktile(kt, Xs0, Ws0, Xs1, Ws1, g0, g1, g3);
+        ktile(kt + 1, Xs1, Ws1, Xs2, Ws2, g1, g2, g0);
+        ktile(kt + 2, Xs2, Ws2, Xs3, Ws3, g2, g3, g1);
+        ktile(kt + 3, Xs3, Ws3, Xs0, Ws0, g3, g0, g2);
     }
 #undef TRN_FETCH_ONE
 #undef TRN_FETCH
