@@ -11,6 +11,14 @@
 // the B operand.  Lane l then holds 16 keys x ONE query, so the per-query normaliser is one scalar per lane,
 // and each lane accumulates its 16 per-key partial sums in registers across all query tiles; the sum over
 // the 32 queries held by different lanes is done once at the end.  No atomics: results are deterministic.
+//
+// Q tiles of 64 queries go straight from global memory into two alternating LDS stages (buffer_load ... lds,
+// XOR-swizzled rows), one barrier per tile.  What the VALU needs per tile besides the scores -- the row
+// normalisers and, for KeyFormer, the wave's 64 x 32 block of fp32 noise, which is the HBM stream that bounds
+// that variant -- is loaded into registers one whole tile ahead, so that a CU always has about 64 KB of noise
+// in flight.  All of these loads are buffer loads with out-of-range zero fill and are issued unconditionally
+// in a fixed order: the wait for a Q stage counts the loads issued behind it.  Masks (causal diagonal, ragged
+// ends) are evaluated only in the blocks that need them (a wave-uniform test).
 #include "common.h"
 
 namespace trn {
@@ -31,12 +39,17 @@ constexpr int CBN = 128;  // keys per workgroup
 constexpr int CBM = 64;   // queries per staged tile
 
 template <int D, bool NOISE>
-__global__ __launch_bounds__(256, 2) void attn_colstats_kernel(const ColArgs a) {
-    constexpr int QP = D + 8;
+__global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const ColArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
     constexpr int NKS = D / 16;
-    __shared__ __attribute__((aligned(16))) half_t Qs[CBM * QP];
+    constexpr int CPR = D / 8;                 // 16-byte chunks per Q row
+    constexpr int RPI = 64 / CPR;              // stage rows covered by one wave-wide 1 KB load
+    constexpr int NI = CBM / (RPI * 4);        // such loads per wave per stage
+    __shared__ __attribute__((aligned(1024))) half_t Qs0[CBM * D];
+    __shared__ __attribute__((aligned(1024))) half_t Qs1[CBM * D];
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, c = lane & 31, h = lane >> 5;
+    const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int BH = a.B * a.Hq;
     const int kt = (int)(blockIdx.x / BH);             // key tile 0 sees the most queries: heaviest first
     const int j = blockIdx.x % BH;
@@ -60,65 +73,117 @@ __global__ __launch_bounds__(256, 2) void attn_colstats_kernel(const ColArgs a) 
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; }
 
-    const half_t* qbase = a.q + b * a.qb + head * a.qh;
-    const float* lrow = a.lse + ((int64_t)b * a.Hq + head) * a.Sq;
-    const float* nbase = NOISE ? a.noise + b * a.nb + head * a.nh : nullptr;
+    // ---- Q stages: direct global -> LDS; queries past the end read as zeros
+    const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.q + b * a.qb + head * a.qh), 0, (int)(((int64_t)(a.Sq - 1) * a.qs + D) * 2), 0x00020000);
+    const int st_row = wave * RPI + lane / CPR;
+    const int st_chunk = (lane % CPR) ^ swz<D>(st_row);
+    const int qvo = (int)(st_row * a.qs * 2) + st_chunk * 16;
+    const int qrow_bytes = (int)(RPI * a.qs * 2), qtile_bytes = (int)(CBM * a.qs * 2);
+#define TRN_FETCH_Q(t_, dst_) fetch_tile<NI, D, 4>(qrs, &dst_[wave * RPI * D], qvo, (t_) * qtile_bytes, qrow_bytes)
+    int qoff[NKS];       // B-operand read: row c (+32 for the second block), logical chunk 2*ks + h
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) qoff[ks] = c * D + (((2 * ks + h) ^ swz<D>(c)) << 3);
+
+    // ---- per-tile register prefetch: row normalisers and noise of the tile's two 32-query blocks
+    const __amdgpu_buffer_rsrc_t lrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.lse + ((int64_t)b * a.Hq + head) * a.Sq), 0, a.Sq * 4, 0x00020000);
+    const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(NOISE ? a.noise + b * a.nb + head * a.nh : a.lse), 0,
+        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
+    const int nvo = NOISE ? (int)((c * a.ns + wkey0 + 4 * h) * 4) : 0;   // lane's query row, first 4 keys of its 16
+    struct Pre { float lse[2]; float4_t g[2][4]; };
+    Pre pre0, pre1;
+    auto prefetch = [&](int t, Pre& p) __attribute__((always_inline)) {
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb)
+            p.lse[qb] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(lrs, c * 4, (t * CBM + qb * 32) * 4, 0));
+        if constexpr (NOISE) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                for (int r4 = 0; r4 < 4; ++r4)
+                    p.g[qb][r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                        nrs, nvo + r4 * 32, (int)((t * CBM + qb * 32) * a.ns * 4), 0));
+        }
+    };
 
     const int first_q = a.causal ? max(0, kv0 - off) : 0;   // earlier queries see none of this tile's keys
-    for (int q0 = (first_q / CBM) * CBM; q0 < a.Sq; q0 += CBM) {
-        __syncthreads();
-#pragma unroll
-        for (int i = 0; i < (CBM * D / 8) / 256; ++i) {
-            const int id = tid + i * 256, row = id / (D / 8), c8 = id % (D / 8);
-            const int qr = q0 + row;
-            uint4_t val = {0u, 0u, 0u, 0u};
-            if (qr < a.Sq) val = *reinterpret_cast<const uint4_t*>(qbase + (int64_t)qr * a.qs + c8 * 8);
-            *reinterpret_cast<uint4_t*>(&Qs[row * QP + c8 * 8]) = val;
-        }
-        __syncthreads();
-        // queries of this tile all earlier than this wave's first key: nothing visible (wave-uniform)
-        if (a.causal && q0 + CBM - 1 + off < wkey0) continue;
+    const int t0 = first_q / CBM, nt = (a.Sq + CBM - 1) / CBM;
 
+    // The VALU part of a 32-query block.  Masked and plain blocks are separate loops (one wave-uniform branch
+    // per block) so that the plain one is 4 instructions per score: fma, exp2, add, fma.
+    auto softmax_sums = [&](const float16_t& acc, int qfirst, float lse, const float4_t (&gq)[4]) __attribute__((always_inline)) {
+        const float lse2 = lse * kLog2e;
+        const bool masked = (qfirst + 31 >= a.Sq) || (wkey0 + 31 >= a.Skv) || (a.causal && wkey0 + 31 > qfirst + off);
+        if (masked) {
+            // last key this lane's query may count, as an offset from the lane's first key (-1: none)
+            const int qrow = qfirst + c;
+            const int last = qrow < a.Sq ? min(a.causal ? qrow + off : a.Skv - 1, a.Skv - 1) - (wkey0 + 4 * h) : -1;
 #pragma unroll
-        for (int qb = 0; qb < CBM / 32; ++qb) {
-            const int qrow = q0 + qb * 32 + c;
-            float16_t acc;
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                half8_t qv = *reinterpret_cast<const half8_t*>(&Qs[(qb * 32 + c) * QP + ks * 16 + 8 * h]);
-                acc = mfma32(kA[ks], qv, acc);
+            for (int r = 0; r < 16; ++r) {
+                float t = __builtin_fmaf(acc[r], a.c1, -lse2);
+                if constexpr (NOISE) t = __builtin_fmaf(gq[r / 4][r % 4], a.c3, t);
+                const float p = (8 * (r / 4) + (r % 4) <= last) ? fast_exp2(t) : 0.f;
+                s1[r] += p;
+                s2[r] = __builtin_fmaf(p, p, s2[r]);
             }
-            const bool qok = qrow < a.Sq;
-            const float lse2 = qok ? lrow[qrow] * kLog2e : 0.f;
-            const float* nrow = NOISE ? nbase + (int64_t)(qok ? qrow : 0) * a.ns : nullptr;
+        } else {
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int key0 = wkey0 + 8 * r4 + 4 * h;
-                float4_t gv = {0.f, 0.f, 0.f, 0.f};
-                if constexpr (NOISE) {
-                    if (qok && key0 < a.Skv && (!a.causal || key0 <= qrow + off)) {
-                        if (key0 + 3 < a.Skv) gv = *reinterpret_cast<const float4_t*>(nrow + key0);
-                        else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) if (key0 + e < a.Skv) gv[e] = nrow[key0 + e];
-                        }
-                    }
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int key = key0 + e;
-                    const bool ok = qok && key < a.Skv && (!a.causal || key <= qrow + off);
-                    float t = __builtin_fmaf(acc[r4 * 4 + e], a.c1, -lse2);
-                    if constexpr (NOISE) t = __builtin_fmaf(gv[e], a.c3, t);
-                    const float p = ok ? fast_exp2(t) : 0.f;
-                    s1[r4 * 4 + e] += p;
-                    s2[r4 * 4 + e] += p * p;
-                }
+            for (int r = 0; r < 16; ++r) {
+                float t = __builtin_fmaf(acc[r], a.c1, -lse2);
+                if constexpr (NOISE) t = __builtin_fmaf(gq[r / 4][r % 4], a.c3, t);
+                const float p = fast_exp2(t);
+                s1[r] += p;
+                s2[r] = __builtin_fmaf(p, p, s2[r]);
             }
         }
+    };
+    // The two 32-query blocks of a tile.  Each block's eight score MFMAs accumulate into one register block (a
+    // dependent chain); all operands of a chain are in registers before it starts, and the second block's are
+    // read while the first chain runs.
+    auto blocks = [&](const half_t* Qc, int q0, const Pre& pc) __attribute__((always_inline)) {
+        // (causal) none of a block's queries sees any of this wave's keys: skip it
+        const bool live0 = !(a.causal && q0 + 31 + off < wkey0), live1 = !(a.causal && q0 + 63 + off < wkey0);
+        if (!live1) return;
+        float16_t acc0, acc1;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+        half8_t qa[NKS];
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[qoff[ks]]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) {
+            acc0 = mfma32(kA[ks], qa[ks], acc0);
+            qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[32 * D + qoff[ks]]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) acc1 = mfma32(kA[ks], qa[ks], acc1);
+        __builtin_amdgcn_sched_barrier(0);
+        if (live0) softmax_sums(acc0, q0, pc.lse[0], pc.g[0]);
+        softmax_sums(acc1, q0 + 32, pc.lse[1], pc.g[1]);
+    };
+    // tile t: its stage has landed once this wave's own share has (everything issued behind it is the
+    // prefetch of the same tile: 2 normaliser loads and, with noise, 8 noise loads) and the others' too
+    auto tile = [&](int t, const half_t* Qc, half_t* Qn, const Pre& pc, Pre& pn) __attribute__((always_inline)) {
+        if constexpr (NOISE) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f72);
+        __builtin_amdgcn_s_barrier();        // (a bare barrier: nothing else in flight needs draining)
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < nt) { TRN_FETCH_Q(t + 1, Qn); prefetch(t + 1, pn); }
+        __builtin_amdgcn_sched_barrier(0);
+        blocks(Qc, t * CBM, pc);
+    };
+    if (t0 < nt) {
+        TRN_FETCH_Q(t0, Qs0);
+        prefetch(t0, pre0);
     }
+    for (int t = t0; t < nt; t += 2) {
+        tile(t, Qs0, Qs1, pre0, pre1);
+        if (t + 1 < nt) tile(t + 1, Qs1, Qs0, pre1, pre0);
+    }
+#undef TRN_FETCH_Q
 
     // sum over the 32 queries held by lanes c = 0..31 (same h), then lane c == 0 of each half writes
     const int64_t obase = ((int64_t)b * a.Hq + head) * a.Skv;
@@ -133,6 +198,7 @@ __global__ __launch_bounds__(256, 2) void attn_colstats_kernel(const ColArgs a) 
             if (a.out_sumsq) a.out_sumsq[obase + key] = y;
         }
     }
+#endif
 }
 
 template <int D, bool NOISE>
@@ -156,6 +222,8 @@ extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, cons
     if (noise) {
         if (!(d->tau > 0.f)) return TRN_E_UNSUPPORTED;
         if (d->noise_stride_s < d->seq_kv) return TRN_E_STRIDE;
+        // one head's noise is addressed with 32-bit byte offsets
+        if ((int64_t)d->seq_q * d->noise_stride_s * 4 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
         if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
             !pitch16(d->noise_stride_b, 4))
             return TRN_E_ALIGN;

@@ -35,32 +35,6 @@ struct AttnArgs {
 
 
 
-// XOR swizzle of the 16-byte chunk index within a tile row, as a function of the row.  Tiles are stored
-// UNPADDED (direct global->LDS loads write 1 KB contiguous per wave instruction), so bank spreading comes from
-// the swizzle: it is a bit permutation of the row's low bits chosen so that (a) 16 consecutive rows read at one
-// logical chunk (the K operand: one 16-byte read per lane, lane = row) and (b) 4 consecutive rows read over 4
-// consecutive chunks (one phase of the transposing V read) both touch every LDS bank exactly once.
-template <int D> __device__ __forceinline__ int swz(int r) {
-    if constexpr (D == 128) return ((r & 3) << 2) | ((r >> 2) & 3);            // 16 chunks per 256-byte row
-    else return (((r >> 1) & 1) << 2) | ((r >> 2) & 3);                        // 8 chunks per 128-byte row
-}
-
-// One wave's share of a K or V stage: NI wave-wide 1 KB loads, global -> LDS without passing through
-// registers.  Load n covers stage rows n*NW*RPI + wave*RPI + lane/CPR (RPI rows of CPR 16-byte chunks); lane i's
-// 16 bytes land at the LDS address of that row group + 16*i.  Which global chunk a lane fetches (vo) decides
-// the swizzle; because the row groups of successive loads are a multiple of 16 rows apart the swizzle is the
-// same for all of them, so ONE per-lane offset serves every load and the rest is wave-uniform (soffset).
-#if defined(__HIP_DEVICE_COMPILE__)
-template <int NI, int D, int NW>
-__device__ __forceinline__ void fetch_tile(__amdgpu_buffer_rsrc_t rs, half_t* dst_wave, int vo, int soff, int row_step_bytes) {
-    constexpr int RPI = 64 / (D / 8);
-#pragma unroll
-    for (int n = 0; n < NI; ++n)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(dst_wave + n * NW * RPI * D),
-                                                 16, vo, soff + n * NW * row_step_bytes, 0, 0);
-}
-#endif
-
 template <int D, int NW, bool NOISE>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer-descriptor types and LDS-load builtins exist in the device pass only;
