@@ -129,7 +129,19 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
     int ntiles = (a.Skv + BN - 1) / BN;
     if (a.causal) ntiles = min(ntiles, (min(q0 + BM - 1, a.Sq - 1) + off) / BN + 1);
 
-    const float* nrow = NOISE ? a.noise + b * a.nb + head * a.nh + (int64_t)qrow_ld * a.ns : nullptr;
+    // KeyFormer noise: this lane's query row, the 4 x 4 keys of its accumulator layout per 32-key block.  It is
+    // the HBM stream that bounds that variant, so each block's 64 bytes per lane are requested two pipeline steps
+    // before they are used (buffer loads: keys or rows past the end read as zeros and are masked anyway).
+    const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(NOISE ? a.noise + b * a.nb + head * a.nh : nullptr), 0,
+        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
+    const int nvo = NOISE ? (int)(((int64_t)qrow_ld * a.ns + 4 * h) * 4) : 0;
+    float4_t gpre0[4], gpre1[4];       // even / odd 32-key blocks: each refilled two blocks ahead, as soon as it is used
+    auto fetch_noise = [&](int key0, float4_t (&gpre)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            gpre[r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(nrs, nvo + r4 * 32, key0 * 4, 0));
+    };
 
     // ---- staging: direct global -> LDS loads.  Buffer descriptors give zero fill for keys past the end
     // (an all-zero V row times P = 0 contributes nothing; garbage could be NaN).
@@ -156,7 +168,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
     // range, fp32 sums), O and l stay relative to the same m so the final O/l and m + log2(l) are unchanged,
     // and the 16*NDB-multiply rescale of O^T runs on the first block or two only instead of on most blocks.
     // Returns whether a rescale is due (wave-uniform) and the candidate max.
-    auto reduce_block = [&](bool masked, float16_t& sx, int key0, float& smax) __attribute__((always_inline)) {
+    auto reduce_block = [&](bool masked, float16_t& sx, int key0, float& smax, float4_t (&gpre)[4]) __attribute__((always_inline)) {
         // `masked` is wave-uniform: the branches below touch only this block's 16 score registers, so the
         // accumulators never meet a control-flow merge.  (Two whole-step variants selected by a branch cost
         // dozens of accumulator register copies per step and broke the in-place MFMA accumulation chains.)
@@ -165,30 +177,19 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
             float16_t z;
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const int k0 = key0 + 8 * r4 + 4 * h;
-                float4_t gv = {0.f, 0.f, 0.f, 0.f};
-                if (masked) {
-                    const bool any_visible = k0 < a.Skv && (!a.causal || k0 <= qrow + off);
-                    if (any_visible) {
-                        if (k0 + 3 < a.Skv) gv = *reinterpret_cast<const float4_t*>(nrow + k0);
-                        else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) if (k0 + e < a.Skv) gv[e] = nrow[k0 + e];
-                        }
-                    }
-                } else {
-                    gv = *reinterpret_cast<const float4_t*>(nrow + k0);
-                }
+                const float4_t gv = gpre[r4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int key = k0 + e;
-                    const bool ok = !masked || (key < a.Skv && (!a.causal || key <= qrow + off));
                     float zz = sx[r4 * 4 + e] * a.c2 + gv[e] * a.c3;
-                    zz = ok ? zz : -INFINITY;
+                    if (masked) {
+                        const int key = key0 + 8 * r4 + 4 * h + e;
+                        zz = (key < a.Skv && (!a.causal || key <= qrow + off)) ? zz : -INFINITY;
+                    }
                     z[r4 * 4 + e] = zz;
                     zmax = fmaxf(zmax, zz);
                 }
             }
+            fetch_noise(key0 + 64, gpre);    // the next block of the same parity, two pipeline steps ahead of its use
             zmax = half_max(zmax);
             if (zmax > -INFINITY) {          // a block can be entirely masked for this row pair
                 float sum = 0.f;
@@ -284,13 +285,14 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
             oacc[i % NDB] = mfma32(va[i % NQ], pB[i / NDB], oacc[i % NDB]);
             if (i + NQ < NS) load_v(i + NQ, i % NQ);
             else ka[i % NQ] = *reinterpret_cast<const half8_t*>(&K2[koff[i + NQ - NS]]);
-            if (i == NS / 2) due = reduce_block(masked_next, sn, key0_next, smax);
+            if (i == NS / 2) due = reduce_block(masked_next, sn, key0_next, smax, SYNC ? gpre1 : gpre0);
             __builtin_amdgcn_sched_barrier(0);
         }
         if (due) rescale(smax);
     };
 
     // ---- prologue: K stages 0 and 1 and V stage 0; scores of block 0; first K operands of block 1 ----
+    if constexpr (NOISE) { fetch_noise(0, gpre0); fetch_noise(32, gpre1); }
     TRN_FETCH_K(0, Ks0);
     TRN_FETCH_V(0, Vs0);
     if (ntiles > 1) TRN_FETCH_K(1, Ks1);
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
 #pragma unroll
         for (int i = 0; i < NQ; ++i) ka[i] = *reinterpret_cast<const half8_t*>(&Ks0[32 * D + koff[i]]);
         float smax;
-        if (reduce_block(true, sA, 0, smax)) rescale(smax);
+        if (reduce_block(true, sA, 0, smax, gpre0)) rescale(smax);
     }
 
     // One 64-key tile jt.  Kc = its own K stage (block 1 still has operands to give), Kn = the next tile's
@@ -315,7 +317,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
     auto tile = [&](int jt, half_t* Kc, const half_t* Kn, const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
         const int kv0 = jt * BN;
         auto handover = [&]() __attribute__((always_inline)) {
-            __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's share of stages Kn and Vc is in LDS
+            // this wave's share of stages Kn and Vc is in LDS: everything but the noise requests of the two
+            // steps since the stages were requested (2 x 4 loads, issued behind them) has returned
+            if constexpr (NOISE) __builtin_amdgcn_s_waitcnt(0x0f78); else __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();                      // ... and everyone's; Kc and Vn have had their last readers
             if (jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
             if (jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
@@ -421,6 +425,8 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     if (noise) {
         if (!(d->tau > 0.f)) return TRN_E_UNSUPPORTED;
         if (d->noise_stride_s < d->seq_kv) return TRN_E_STRIDE;
+        // one head's noise is addressed with 32-bit byte offsets
+        if ((int64_t)d->seq_q * d->noise_stride_s * 4 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
         if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
             !pitch16(d->noise_stride_b, 4))
             return TRN_E_ALIGN;
