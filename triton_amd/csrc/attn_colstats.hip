@@ -171,7 +171,11 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
         if constexpr (NOISE) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f72);
         __builtin_amdgcn_s_barrier();        // (a bare barrier: nothing else in flight needs draining)
         __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < nt) { TRN_FETCH_Q(t + 1, Qn); prefetch(t + 1, pn); }
+        // unconditional (past the last tile everything reads as zeros into a stage nobody uses): the compiler sizes
+        // its waits for the prefetched registers by the loads it KNOWS follow them, and a conditional load counts
+        // as absent, which would make every use of a prefetched value drain the stage refill as well
+        TRN_FETCH_Q(t + 1, Qn);
+        prefetch(t + 1, pn);
         __builtin_amdgcn_sched_barrier(0);
         blocks(Qc, t * CBM, pc);
     };
@@ -179,6 +183,11 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
         TRN_FETCH_Q(t0, Qs0);
         prefetch(t0, pre0);
     }
+    // Pin the arrival of the K rows here, ahead of the loop.  Left to the first MFMA that reads them, the wait the
+    // compiler inserts sits inside the loop body and, being conservative across the back edge, drains the stage and
+    // prefetch loads of every iteration.
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) asm volatile("" ::"v"(kA[ks]));
     for (int t = t0; t < nt; t += 2) {
         tile(t, Qs0, Qs1, pre0, pre1);
         if (t + 1 < nt) tile(t + 1, Qs1, Qs0, pre1, pre0);

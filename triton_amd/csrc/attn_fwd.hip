@@ -321,8 +321,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
             // steps since the stages were requested (2 x 4 loads, issued behind them) has returned
             if constexpr (NOISE) __builtin_amdgcn_s_waitcnt(0x0f78); else __builtin_amdgcn_s_waitcnt(0x0f70);
             __syncthreads();                      // ... and everyone's; Kc and Vn have had their last readers
-            if (jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
-            if (jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
+            // With noise in flight the refills are issued unconditionally (tiles past the end just fill stages
+            // nobody reads): the compiler sizes its waits for the noise registers by the loads it KNOWS follow
+            // them, and a conditional load counts as absent -- every noise use would drain the refills too.
+            if (NOISE || jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
+            if (NOISE || jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
         };
         auto none = [&]() __attribute__((always_inline)) {};
         // (Past the last tile a K stage holds stale rows; scores computed from them are masked away.)
