@@ -1,0 +1,181 @@
+"""GPU checks at the benchmarked (full) sizes: size-independent properties of the domain over the whole problem, and
+oracle parity on a sample of heads (the CPU oracle does one S=4096 head in a fraction of a second; all 32 would take
+minutes).  Tolerances as everywhere: fp16 attention outputs atol 2e-2 / rtol 1e-2, RMSNorm 1e-3 relative, fp32 key
+scores 1e-3 relative."""
+import pytest
+import torch
+
+from oracle import ref
+from triton_amd import configs
+
+pytestmark = pytest.mark.gpu
+
+
+def close(got, want, atol=2e-2, rtol=1e-2):
+    got = got.float().cpu(); want = want.float().cpu()
+    err = (got - want).abs()
+    bad = err > atol + rtol * want.abs()
+    assert not bad.any(), f"{int(bad.sum())} off; max abs err {err.max():.4g}"
+
+
+def llama_qkv(S, seed=42):
+    c = configs.LLAMA
+    g = torch.Generator().manual_seed(seed)
+    q = ref.randn_half((1, c["n_heads"], S, c["head_dim"]), g)
+    k = ref.randn_half((1, c["n_kv_heads"], S, c["head_dim"]), g)
+    v = ref.randn_half((1, c["n_kv_heads"], S, c["head_dim"]), g)
+    return q, k, v
+
+
+def head_slice(q, k, v, h, group):
+    """Query head h with its KV head, as a 1-head problem for the oracle."""
+    return q[:, h:h + 1], k[:, h // group:h // group + 1], v[:, h // group:h // group + 1]
+
+
+def test_vanilla_llama_s4096_sampled_parity_and_properties():
+    from triton_amd import ops
+    S = configs.VANILLA["seq"]; D = configs.LLAMA["head_dim"]; scale = D ** -0.5
+    q, k, v = llama_qkv(S)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(1, 32, S, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, True, lse=lse)
+    torch.cuda.synchronize()
+    for h in (0, 13, 31):                                   # first, a middle and the last query head
+        wo, wl = ref.attention(*head_slice(q, k, v, h, 4), scale, True, return_lse=True)
+        close(o[:, h:h + 1], wo); close(lse[:, h:h + 1], wl, atol=1e-3, rtol=1e-3)
+    # a convex combination of V rows: constant V columns come back unchanged, whatever the weights
+    vc = torch.empty_like(vd); vc[:] = torch.linspace(-2, 2, D, device="cuda", dtype=torch.float16)
+    oc = torch.zeros_like(qd)
+    ops.attention(qd, kd, vc, oc, scale, True)
+    assert (oc.float() - vc[0, 0, 0].float()).abs().max() < 4e-3
+    # linear in V
+    g = torch.Generator().manual_seed(3)
+    v2 = ref.randn_half(tuple(v.shape), g).cuda()
+    o2 = torch.zeros_like(qd); o12 = torch.zeros_like(qd)
+    ops.attention(qd, kd, v2, o2, scale, True)
+    ops.attention(qd, kd, (vd.float() + v2.float()).half(), o12, scale, True)
+    close(o12, o.float() + o2.float(), atol=3e-2)
+    # causal: queries before position t never see keys / values from t on.  Bit-identical outputs when t is a
+    # multiple of the 32 queries a wave owns (within a wave the moment of a running-max update, hence the rounding,
+    # is shared by its rows); equal within tolerance for any t.
+    t = 2560
+    k3, v3 = kd.clone(), vd.clone()
+    k3[:, :, t:] = 7.0; v3[:, :, t:] = -9.0
+    o3 = torch.zeros_like(qd)
+    ops.attention(qd, k3, v3, o3, scale, True)
+    torch.cuda.synchronize()
+    assert torch.equal(o3[:, :, :t], o[:, :, :t])
+    assert not torch.equal(o3[:, :, t:], o[:, :, t:])
+    t = 2500
+    k3[:, :, t:2560] = 7.0; v3[:, :, t:2560] = -9.0
+    ops.attention(qd, k3, v3, o3, scale, True)
+    torch.cuda.synchronize()
+    close(o3[:, :, :t], o[:, :, :t])
+
+
+def test_roco_and_keyformer_llama_s4096_invariants_and_sampled_parity():
+    from triton_amd import ops
+    S = configs.ROCO["seq"]; D = configs.LLAMA["head_dim"]; scale = D ** -0.5
+    q, k, v = llama_qkv(S, seed=5)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(1, 32, S, device="cuda")
+    s1 = torch.full((1, 32, S), -1.0, device="cuda"); s2 = torch.full((1, 32, S), -1.0, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, True, lse=lse)
+    ops.attention_colstats(qd, kd, lse, scale, True, s1, s2)
+    torch.cuda.synchronize()
+    # every probability row sums to 1: the column sums of a head add up to the number of queries
+    assert torch.allclose(s1.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
+    assert (s2 >= 0).all() and (s2 <= s1 * (1 + 1e-5) + 1e-6).all()      # 0 <= p^2 <= p
+    assert torch.isfinite(s1).all() and torch.isfinite(s2).all()
+    for h in (2, 30):
+        qh, kh, vh = head_slice(q, k, v, h, 4)
+        wo, w1, w2 = ref.roco(qh, kh, vh, scale, True)
+        err1 = (s1[:, h:h + 1].cpu() - w1).abs(); err2 = (s2[:, h:h + 1].cpu() - w2).abs()
+        assert (err1 <= 1e-5 + 1e-3 * w1.abs()).all() and (err2 <= 1e-5 + 1e-3 * w2.abs()).all()
+    # KeyFormer with zero noise and tau = 1 is RoCo's column sum; with noise the scores still add up to S
+    noise = torch.zeros(1, 32, S, S, device="cuda")
+    lsep = torch.zeros(1, 32, S, device="cuda"); score = torch.full((1, 32, S), -1.0, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, True, noise=noise, tau=1.0, lse_pert=lsep)
+    ops.attention_colstats(qd, kd, lsep, scale, True, score, None, noise=noise, tau=1.0)
+    torch.cuda.synchronize()
+    # (the plain row sum is taken over the fp16-rounded probabilities that multiply V, the perturbed one in fp32)
+    assert torch.allclose(lsep, lse, rtol=1e-3, atol=1e-3)
+    assert torch.allclose(score, s1, rtol=1e-3, atol=1e-5)
+    # Gumbel noise drawn on the device for the whole problem (properties), from the seeded host generator for the
+    # sampled head (parity: both sides consume the same bits)
+    u = torch.rand(1, 32, S, S, device="cuda").clamp_(1e-10, 1 - 1e-7)
+    noise = -torch.log(-torch.log(u)); del u
+    h = 17
+    noise[:, h] = ref.gumbel_noise((1, 1, S, S), configs.KEYFORMER["noise_seed"])[:, 0].cuda()
+    ops.attention(qd, kd, vd, o, scale, True, noise=noise, tau=1.0, lse_pert=lsep)
+    ops.attention_colstats(qd, kd, lsep, scale, True, score, None, noise=noise, tau=1.0)
+    torch.cuda.synchronize()
+    assert torch.allclose(score.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
+    qh, kh, vh = head_slice(q, k, v, h, 4)
+    wo, wscore = ref.keyformer(qh, kh, vh, noise[:, h:h + 1].cpu(), scale, 1.0, True)
+    err = (score[:, h:h + 1].cpu() - wscore).abs()
+    assert (err <= 1e-5 + 1e-3 * wscore.abs()).all()
+    close(o[:, h:h + 1], wo)
+
+
+def test_qknorm_falcon_s2048_sampled_parity_and_scale_invariance():
+    from triton_amd import modules
+    c = configs.QKNORM; S, H, D = c["seq"], c["n_heads"], c["head_dim"]
+    g = torch.Generator().manual_seed(11)
+    q = ref.randn_half((1, H, S, D), g); k = ref.randn_half((1, 1, S, D), g); v = ref.randn_half((1, 1, S, D), g)
+    gq = ref.randn_half((D,), g, 1.0, 0.02); gk = ref.randn_half((D,), g, 1.0, 0.02)
+    mod = modules.get("qknorm", eps=c["eps"])
+    names = mod.TENSOR_PARAMS
+
+    def run(qq, kk):
+        t = dict(Q=qq.cuda(), K=kk.cuda(), V=v.cuda(), O=torch.zeros(1, H, S, D, dtype=torch.float16, device="cuda"),
+                 gamma_q=gq.cuda(), gamma_k=gk.cuda())
+        mod.forward(*[t[n] for n in names])
+        torch.cuda.synchronize()
+        return t["O"]
+
+    o = run(q, k)
+    for h in (0, 35, 70):
+        want = ref.qknorm_attention(q[:, h:h + 1], k, v, gq, gk, c["eps"], D ** -0.5, True)
+        close(o[:, h:h + 1], want)
+    # per-head RMSNorm makes the result (almost: eps) independent of the scale of Q and of K
+    o4 = run((q.float() * 4).half(), (k.float() * 0.25).half())
+    close(o4, o, atol=2e-2)
+
+
+def test_prenorm_block_llama_s2048_sampled_parity():
+    from triton_amd import modules
+    c = configs.PRENORM; S, N, D = c["seq"], c["hidden"], c["head_dim"]
+    nkv = c["n_kv_heads"] * D
+    g = torch.Generator().manual_seed(21)
+    x = ref.randn_half((1, S, N), g); gamma = ref.randn_half((N,), g, 1.0, 0.02)
+    wq = ref.randn_half((N, N), g, 0, 0.02); wk = ref.randn_half((N, nkv), g, 0, 0.02); wv = ref.randn_half((N, nkv), g, 0, 0.02)
+    mod = modules.get("prenorm", head_dim=D, eps=c["eps"])
+    t = dict(X=x.cuda(), gamma=gamma.cuda(), WQ=wq.cuda(), WK=wk.cuda(), WV=wv.cuda(),
+             O=torch.zeros(1, S, N, dtype=torch.float16, device="cuda"))
+    mod.forward(*[t[n] for n in mod.TENSOR_PARAMS])
+    torch.cuda.synchronize()
+    want = ref.prenorm_block(x, gamma, wq, wk, wv, D, c["eps"], D ** -0.5, True)     # [1, S, N] token-major
+    close(t["O"], want)
+    # RMSNorm makes the block independent of the scale of X (up to eps)
+    t2 = dict(t, X=(x.float() * 8).half().cuda(), O=torch.zeros_like(t["O"]))
+    mod.forward(*[t2[n] for n in mod.TENSOR_PARAMS])
+    torch.cuda.synchronize()
+    close(t2["O"], t["O"])
+
+
+def test_rmsnorm_4096_square_invariants():
+    from triton_amd import ops
+    c = configs.RMSNORM
+    g = torch.Generator().manual_seed(42)
+    x = ref.randn_half((c["rows"], c["cols"]), g).cuda()
+    y = torch.empty_like(x); y2 = torch.empty_like(x)
+    ops.rmsnorm(x, None, y, 0.0)
+    ops.rmsnorm((x.float() * 3).half(), None, y2, 0.0)
+    torch.cuda.synchronize()
+    ms = y.float().pow(2).mean(-1)
+    assert torch.allclose(ms, torch.ones_like(ms), rtol=2e-3)                 # unit mean square at eps = 0, gamma = 1
+    assert (y.float() - y2.float()).abs().max() <= 2e-3 * y.float().abs().max()   # scale-equivariant
+    ops.rmsnorm(y, None, y2, 0.0)                                              # idempotent up to fp16 rounding
+    torch.cuda.synchronize()
+    assert (y.float() - y2.float()).abs().max() <= 2e-3 * y.float().abs().max()
