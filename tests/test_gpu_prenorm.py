@@ -24,7 +24,10 @@ def weights(g, K, nq, nkv, std=0.02):
                                               (1, 64, 64, 64, 64, True), (16, 4544, 4544, 64, 64, True),
                                               # 256 x 256 tiling (>= 128 of its tiles): ragged tokens and hidden,
                                               # a nearly empty K/V panel, no norm
-                                              (1000, 520, 6144, 1024, 128, True), (300, 200, 16384, 64, 64, False)])
+                                              (1000, 520, 6144, 1024, 128, True), (300, 200, 16384, 64, 64, False),
+                                              # at most 32 tokens: the weight-streaming tiling (four waves split hidden)
+                                              (32, 520, 1024, 256, 128, True), (5, 72, 192, 64, 64, True),
+                                              (17, 8192, 256, 128, 128, True), (33, 520, 256, 128, 128, True)])
 def test_qkv_projection_parity(T, K, nq, nkv, D, norm):
     from triton_amd import ops
     g = torch.Generator().manual_seed(42)
@@ -61,6 +64,7 @@ def test_projection_into_kv_cache_rows():
 
 
 @pytest.mark.parametrize("T,K,nq,nkv,D", [(200, 136, 256, 64, 64),         # 128 x 128 tiling
+                                         (20, 136, 320, 64, 64),          # weight-streaming tiling
                                          (600, 136, 5120, 512, 128)])      # 256 x 256 tiling
 def test_projection_reads_and_writes_stay_inside_its_views(T, K, nq, nkv, D):
     """Operands are padded views cut out of NaN-filled buffers, hidden and tokens are ragged: a tile load that strays

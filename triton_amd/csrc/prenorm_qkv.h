@@ -27,4 +27,7 @@ __device__ __forceinline__ int wswz(int r) { return ((r & 3) << 2) | ((r >> 2) &
 int launch_prenorm_qkv_wide(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream);
 int64_t prenorm_qkv_wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv);
 
+// At most 32 tokens: 64-column panels streamed by four waves that split the contraction (prenorm_qkv_skinny.hip).
+int launch_prenorm_qkv_skinny(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream);
+
 }  // namespace trn

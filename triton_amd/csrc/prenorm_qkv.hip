@@ -238,6 +238,8 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0};
     a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, 0};
     a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, 0};
+    // a handful of tokens (decode): the weight stream is everything
+    if (tokens <= 32) return launch_prenorm_qkv_skinny(a, n_q, n_kv, (hipStream_t)stream);
     // 256 x 256 tiles once they alone occupy at least half of the 256 CUs; 128 x 128 tiles below that (decode
     // and short prefills, where the number of workgroups matters more than the work per staged byte)
     if (prenorm_qkv_wide_tiles(tokens, n_q, n_kv) >= 128) return launch_prenorm_qkv_wide(a, n_q, n_kv, (hipStream_t)stream);
