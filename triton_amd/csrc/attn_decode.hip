@@ -1,0 +1,233 @@
+// Attention forward for at most 32 queries per head (decode-append: a few new tokens against a long cache).
+//
+// With so few queries there is one 32-query MFMA block per head and the kernel is a stream of K and V through HBM.
+// One workgroup per (batch, head); its eight waves take the 32-key blocks round-robin, each with its own running
+// max / normaliser / O^T accumulator, and the eight partial results are merged through LDS at the end (the usual
+// log-sum-exp merge).  Formulation and register layouts are those of the prefill kernel: S^T = K Q^T with Q^T
+// resident in registers, P^T taken from the S^T accumulator, V^T via the transposing LDS read.  K rows are what the
+// A operand wants as they lie in memory, so K goes straight from global memory into registers (one block ahead);
+// V goes global -> LDS into the wave's private two-stage ring.  Nothing in the loop is shared between waves, so the
+// loop has no barrier; every load is issued unconditionally (blocks past the end read zeros, which are masked) so
+// that the waits can be counted.
+#include "attn.h"
+
+namespace trn {
+
+constexpr int DNW = 8;    // waves per workgroup
+
+template <int D>
+__global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs a) {
+#if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
+    constexpr int NS = D / 16;    // k-steps of S^T = K Q^T; also (2 key halves) x (D/32) MFMAs of P V
+    constexpr int NDB = D / 32;
+    constexpr int CPR = D / 8;    // 16-byte chunks per row
+    constexpr int RPI = 64 / CPR; // rows per wave-wide 1 KB load
+    constexpr int NI = 32 / RPI;  // such loads per 32-key V block
+    // two V stages (each holds the eight waves' private parts), as two arrays: LDS reads are ordered after
+    // outstanding global->LDS loads that may alias them, and only distinct variables are provably disjoint
+    __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * D];
+    __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * D];
+    __shared__ float st_m[DNW][32], st_l[DNW][32];
+
+    const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int j = blockIdx.x;
+    const int G = a.Hq / a.Hkv, nkv = a.B * a.Hkv;
+    const int kvslot = j % nkv, g = j / nkv;
+    const int b = kvslot / a.Hkv, kvh = kvslot % a.Hkv, head = kvh * G + g;
+    const int off = a.Skv - a.Sq;                       // causal: query i sees keys <= i + off
+    const int qrow = c;                                 // this lane's query
+    const int qrow_ld = qrow < a.Sq ? qrow : a.Sq - 1;
+
+    // ---- Q^T B-operands: lane holds Q[qrow][ks*16 + 8h .. +7]; optional fused per-head RMSNorm of the row
+    half8_t qB[NS];
+    {
+        const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * h;
+#pragma unroll
+        for (int ks = 0; ks < NS; ++ks) qB[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 16);
+        if (a.q_norm) {
+            float ss = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < NS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { float f = (float)qB[ks][e]; ss += f * f; }
+            ss = half_sum(ss);
+            const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
+#pragma unroll
+            for (int ks = 0; ks < NS; ++ks) {
+                half8_t gq;
+                if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 16 + 8 * h);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float y = (float)qB[ks][e] * rstd;
+                    if (a.gamma_q) y = (float)gq[e] * y;
+                    qB[ks][e] = (half_t)y;
+                }
+            }
+        }
+    }
+    // pin the arrival of Q here: left to the first MFMA in the loop, the compiler's wait would sit in the loop body
+#pragma unroll
+    for (int ks = 0; ks < NS; ++ks) asm volatile("" ::"v"(qB[ks]));
+
+    // ---- K: block rows straight into registers as A operands (lane: key c of the block, columns ks*16 + 8h ..)
+    const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.k + b * a.kb + kvh * a.kh), 0, (int)(((int64_t)(a.Skv - 1) * a.ks + D) * 2), 0x00020000);
+    const int kvo = (int)(c * a.ks * 2) + 16 * h;
+    const int kblk_bytes = (int)(32 * a.ks * 2);
+    auto fetch_k = [&](int blk, half8_t (&ka)[NS]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int ks = 0; ks < NS; ++ks)
+            ka[ks] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvo + ks * 32, blk * kblk_bytes, 0));
+    };
+    // ---- V: block rows global -> LDS, chunk c of row r stored at c ^ swz<D>(r); load n covers rows n*RPI + lane/CPR
+    const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(a.v + b * a.vb + kvh * a.vh), 0, (int)(((int64_t)(a.Skv - 1) * a.vs + D) * 2), 0x00020000);
+    int vvo[NI];
+#pragma unroll
+    for (int n = 0; n < NI; ++n) {
+        const int r = n * RPI + lane / CPR;
+        vvo[n] = (int)(r * a.vs * 2) + (((lane % CPR) ^ swz<D>(r)) << 4);
+    }
+    const int vblk_bytes = (int)(32 * a.vs * 2);
+#define TRN_FETCH_V(blk_, dst_)                                                                                  \
+    _Pragma("unroll") for (int n_ = 0; n_ < NI; ++n_) __builtin_amdgcn_raw_ptr_buffer_load_lds(                  \
+        vrs, (__attribute__((address_space(3))) void*)(&dst_[wave * 32 * D + n_ * RPI * D]), 16, vvo[n_],        \
+        (blk_) * vblk_bytes, 0, 0)
+    // V^T operand through the transposing read (as in the prefill kernel): rows 4h + (lane%16)/4 [+8] of a 16-key half
+    int voff_lo[NDB], voff_hi[NDB];
+    {
+        const int rl = 4 * h + ((lane & 15) >> 2), rh = rl + 8;
+        const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), sub = (lane & 1) * 4;
+#pragma unroll
+        for (int db = 0; db < NDB; ++db) {
+            voff_lo[db] = wave * 32 * D + rl * D + (((db * 4 + lc) ^ swz<D>(rl)) << 3) + sub;
+            voff_hi[db] = wave * 32 * D + rh * D + (((db * 4 + lc) ^ swz<D>(rh)) << 3) + sub;
+        }
+    }
+
+    float16_t oacc[NDB];
+#pragma unroll
+    for (int i = 0; i < NDB; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
+    float m = -INFINITY, l = 0.f;       // running max (log2 domain, shared by the lane pair) and this lane's partial sum
+
+    const int nblk = (a.Skv + 31) / 32;
+    const int nmine = (nblk - wave + DNW - 1) / DNW;          // blocks wave, wave + 8, ...
+    half8_t ka0[NS], ka1[NS];
+
+    // One 32-key block whose K is in kc and whose V is in stage Vc; the next block's loads go to kn / Vn first.
+    auto block = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
+        const int blk = wave + it * DNW, key0 = blk * 32;
+        fetch_k(blk + DNW, kn);
+        TRN_FETCH_V(blk + DNW, Vn);
+        float16_t s;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NS; ++ks) s = mfma32(kc[ks], qB[ks], s);
+        // mask (wave-uniform test), block max, running max, probabilities
+        const bool masked = (key0 + 32 > a.Skv) || (a.causal && key0 + 31 > off);
+        if (masked) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
+                s[r] = (key < a.Skv && (!a.causal || key <= qrow + off)) ? s[r] : -INFINITY;
+            }
+        }
+        float smax = s[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) smax = fmaxf(smax, s[r]);
+        smax = half_max(smax) * a.c1;
+        const float mnew = fmaxf(m, smax);
+        const float mref = mnew == -INFINITY ? 0.f : mnew;     // a row can see nothing of a block
+        const float alpha = fast_exp2(m - mref);               // m = -inf: 0
+        const half2_t ones = {(half_t)1.f, (half_t)1.f};
+        half8_t pB[2];
+        l *= alpha;
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+            const half2_t pp = {(half_t)fast_exp2(__builtin_fmaf(s[r], a.c1, -mref)),
+                                (half_t)fast_exp2(__builtin_fmaf(s[r + 1], a.c1, -mref))};
+            l = __builtin_amdgcn_fdot2(pp, ones, l, false);    // the row sum of exactly the values that multiply V
+            pB[r / 8][r % 8] = pp[0]; pB[r / 8][r % 8 + 1] = pp[1];
+        }
+#pragma unroll
+        for (int i = 0; i < NDB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        m = mnew;
+        // this block's V has landed: behind it only the next block's NS + NI requests were issued
+        __builtin_amdgcn_s_waitcnt(0x0f70 | ((NS + NI) & 15) | (((NS + NI) >> 4) << 14));
+#pragma unroll
+        for (int i = 0; i < NS; ++i) {
+            const half_t* vp = Vc + 16 * (i / NDB) * D;
+            const half4_t lo = lds_read_tr16(vp + voff_lo[i % NDB]);
+            const half4_t hi = lds_read_tr16(vp + voff_hi[i % NDB]);
+            const half8_t va = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            oacc[i % NDB] = mfma32(va, pB[i / NDB], oacc[i % NDB]);
+        }
+    };
+    fetch_k(wave, ka0);
+    TRN_FETCH_V(wave, Vs0);
+    for (int it = 0; it < nmine; it += 2) {
+        block(it, ka0, ka1, Vs0, Vs1);
+        if (it + 1 < nmine) block(it + 1, ka1, ka0, Vs1, Vs0);
+    }
+#undef TRN_FETCH_V
+
+    // ---- merge the eight waves' (m, l, O^T) through LDS.  Partial O^T as float4 quads [d/4][query]: the first half
+    // of head_dim in this wave's part of Vs0, the second half in its part of Vs1 (each exactly 32 * D/2 floats).
+    l = half_sum(l);
+    __builtin_amdgcn_s_waitcnt(0x0f70);                 // the look-ahead requests past the end have landed too
+    if (h == 0) { st_m[wave][c] = m; st_l[wave][c] = l; }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db) {
+        float4_t* part = reinterpret_cast<float4_t*>((db < NDB / 2 ? Vs0 : Vs1) + wave * 32 * D);
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            part[((db % (NDB / 2)) * 8 + 2 * r4 + h) * 32 + c] =
+                float4_t{oacc[db][r4 * 4], oacc[db][r4 * 4 + 1], oacc[db][r4 * 4 + 2], oacc[db][r4 * 4 + 3]};
+    }
+    __syncthreads();
+    {
+        const int q = tid & 31, dg = tid >> 5;            // 16 groups of threads share out the D/4 quads of a query
+        float mstar = st_m[0][q];
+#pragma unroll
+        for (int w = 1; w < DNW; ++w) mstar = fmaxf(mstar, st_m[w][q]);
+        float wgt[DNW], L = 0.f;
+#pragma unroll
+        for (int w = 0; w < DNW; ++w) { wgt[w] = fast_exp2(st_m[w][q] - mstar); L += st_l[w][q] * wgt[w]; }   // idle waves: m = -inf, weight 0
+        const float inv = 1.0f / L;
+        half_t* orow = a.o + b * a.ob + head * a.oh + (int64_t)q * a.os;
+#pragma unroll
+        for (int qi = 0; qi < (D / 4) / 16; ++qi) {
+            const int quad = dg + 16 * qi;                // d = 4*quad .. +3
+            const half_t* base = quad < D / 8 ? Vs0 : Vs1;
+            const int ql = quad % (D / 8);
+            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int w = 0; w < DNW; ++w) {
+                const float4_t v = reinterpret_cast<const float4_t*>(base + w * 32 * D)[ql * 32 + q];
+                acc += v * wgt[w];
+            }
+            if (q < a.Sq) {
+                const half4_t ov = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv), (half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
+                *reinterpret_cast<half4_t*>(orow + 4 * quad) = ov;
+            }
+        }
+        if (dg == 0 && q < a.Sq && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
+    }
+#endif
+}
+
+hipError_t launch_attn_decode(const AttnArgs& a, int head_dim, hipStream_t stream) {
+    const int64_t grid = (int64_t)a.B * a.Hq;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
+    if (head_dim == 128) hipLaunchKernelGGL(attn_decode_kernel<128>, dim3((unsigned)grid), dim3(DNW * 64), 0, stream, a);
+    else hipLaunchKernelGGL(attn_decode_kernel<64>, dim3((unsigned)grid), dim3(DNW * 64), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace trn

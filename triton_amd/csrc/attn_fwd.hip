@@ -17,23 +17,10 @@
 // Grid: one workgroup per (query tile, batch, head), heaviest (latest) query tiles first; consecutive
 // workgroup ids map to different KV heads so that the query heads sharing a KV head land on the same XCD
 // (ids are dealt round-robin to the 8 XCDs) and hit its L2.
-#include "common.h"
+#include "attn.h"
 #include <type_traits>
 
 namespace trn {
-
-struct AttnArgs {
-    const half_t* q; const half_t* k; const half_t* v; half_t* o;
-    float* lse; const half_t* gamma_q; const float* noise; float* lse_pert;
-    int B, Hq, Hkv, Sq, Skv, n_qtiles;
-    int64_t qb, qh, qs, kb, kh, ks, vb, vh, vs, ob, oh, os, nb, nh, ns;
-    float c1;      // scale * log2(e)                    : plain scores in the log2 domain
-    float c2, c3;  // scale*log2(e)/tau, log2(e)/tau     : perturbed scores  z2 = s*c2 + g*c3
-    float q_eps;
-    int causal, q_norm;
-};
-
-
 
 template <int D, int NW, bool NOISE>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(const AttnArgs a) {
@@ -453,6 +440,8 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
         return TRN_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
+    // a handful of queries per head (decode): one workgroup per head, its waves split the keys
+    if (!noise && d->seq_q <= 32) return launch_attn_decode(a, d->head_dim, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
     // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
     // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
     // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to
