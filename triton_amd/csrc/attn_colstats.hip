@@ -36,7 +36,7 @@ struct ColArgs {
 };
 
 constexpr int CBN = 128;  // keys per workgroup
-constexpr int CBM = 64;   // queries per staged tile
+[[maybe_unused]] constexpr int CBM = 64;   // queries per staged tile
 
 template <int D, bool NOISE>
 __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const ColArgs a) {

@@ -14,7 +14,7 @@
 
 namespace trn {
 
-constexpr int SN = 64, SK = 32, SS = 6;      // panel columns, contraction rows per stage, stages per wave
+[[maybe_unused]] constexpr int SN = 64, SK = 32, SS = 6;      // panel columns, contraction rows per stage, stages per wave
 
 __global__ __launch_bounds__(256, 1) void prenorm_qkv_skinny_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only

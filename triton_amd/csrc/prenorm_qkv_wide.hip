@@ -18,7 +18,7 @@
 
 namespace trn {
 
-constexpr int WM = 256, WN = 256, WK = 32;
+[[maybe_unused]] constexpr int WM = 256, WN = 256, WK = 32;
 
 __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
