@@ -445,10 +445,10 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
     // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
     // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to
-    // n_qtiles x, so at least two rounds are needed to balance (measured: +2.3 % at 512 wide workgroups).  Otherwise 4 waves x 32 (two workgroups per CU).
+    // n_qtiles x, so at least two rounds are needed to balance (measured at 512 wide workgroups: +2.3 % with head_dim 128, -10 % with 64, which is VALU- rather than power-bound).  Otherwise 4 waves x 32 (two workgroups per CU).
 #ifndef TRN_FORCE_NW
     const int64_t n_wide = (int64_t)((d->seq_q + 255) / 256) * d->batch * d->n_q_heads;
-    const bool wide = n_wide >= (d->causal ? 512 : 256);
+    const bool wide = n_wide >= (!d->causal ? 256 : d->head_dim == 128 ? 512 : 1024);
 #else
     const bool wide = TRN_FORCE_NW == 8;
 #endif
