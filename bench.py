@@ -35,7 +35,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="default",
-                    help="default (vanilla headline + rmsnorm), all, or one of vanilla rmsnorm prenorm qknorm keyformer roco")
+                    help="default (vanilla headline + rmsnorm), all, or one of vanilla rmsnorm prenorm qknorm keyformer roco decode")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
     ap.add_argument("--calibrate", action="store_true",
@@ -205,6 +205,31 @@ def bench_variant(name, steps, warmup):
     return out
 
 
+def bench_decode(steps, warmup):
+    """The reference's own problem form (M new tokens projected, appended to the caches, attended over P+M keys;
+    convert_eval_rms.py:33-60) timed the way its drivers time a candidate: one forward per graph replay.
+    Microseconds per forward for each variant at the Llama and Falcon widths, and the bytes that must move."""
+    import torch
+    from triton_amd import configs, modules
+    out = {}
+    for name, cfg in (("llama", configs.DECODE_LLAMA), ("falcon", configs.DECODE_FALCON)):
+        M, N, D, H, P = cfg["M"], cfg["N"], cfg["D"], cfg["H"], cfg["P"]
+        g = torch.Generator(device="cuda").manual_seed(42)
+        rnd = lambda *shape: torch.randn(*shape, device="cuda", generator=g).clamp_(-1, 1).mul_(0.01).half()
+        t = dict(X=rnd(M, N), WQ=rnd(N, N), WK=rnd(N, N), WV=rnd(N, N), K_cache=rnd(H, P + M, D), V_cache=rnd(H, P + M, D),
+                 O2=torch.zeros(M, N, dtype=torch.float16, device="cuda"),
+                 noise=torch.randn(H, M, P + M, device="cuda", generator=g).half())
+        for c in ("C_out", "C_out1", "C_out2"):
+            t[c] = torch.zeros(H, P + M, dtype=torch.float16, device="cuda")
+        res = {"weights_and_cache_bytes": 3 * N * N * 2 + 2 * H * (P + M) * D * 2}
+        for v in ("vanilla", "prenorm", "qknorm", "keyformer", "roco"):
+            m = modules.get(v, "decode", head_dim=D)
+            _, ev = graph_timed(m, t, steps, warmup, per_graph=1)
+            res[v + "_us"] = round(ev * 1e3, 2)
+        out[name] = res
+    return out
+
+
 def mfma_ceiling():
     """TFLOP/s of the MFMA-only yardstick kernel with all-zero and with random fp16 operands."""
     import torch
@@ -281,6 +306,8 @@ def main():
         if wl in ("all", name):
             extra[name] = bench_variant(name, max(a.steps // 4, 10), a.warmup)
             torch.cuda.empty_cache()
+    if wl in ("all", "decode"):
+        extra["decode_append_M16_P1024"] = bench_decode(100, a.warmup)
     if van is None:                       # a single non-headline workload was asked for
         print(json.dumps({"workload": wl, **extra}))
         return
@@ -321,6 +348,8 @@ def main():
     for name in ("prenorm", "qknorm", "keyformer", "roco"):
         if name in extra:
             line[name] = {k: (round(v, 4) if isinstance(v, float) else v) for k, v in extra[name].items()}
+    if "decode_append_M16_P1024" in extra:
+        line["decode_append_M16_P1024"] = extra["decode_append_M16_P1024"]
     if not a.no_cpu:
         line["cpu_baseline"] = cpu_baseline(*van["tensors"], a.cpu_seconds)
         line["cpu_baseline"]["value"] = round(line["cpu_baseline"]["value"], 4)
