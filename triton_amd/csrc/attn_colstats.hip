@@ -232,11 +232,14 @@ extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, cons
         if (!(d->tau > 0.f)) return TRN_E_UNSUPPORTED;
         if (d->noise_stride_s < d->seq_kv) return TRN_E_STRIDE;
         // one head's noise is addressed with 32-bit byte offsets
-        if ((int64_t)d->seq_q * d->noise_stride_s * 4 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
+        if (((int64_t)d->seq_q + 128) * d->noise_stride_s * 4 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
         if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
             !pitch16(d->noise_stride_b, 4))
             return TRN_E_ALIGN;
     }
+    // Q tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base (with room for the tile requested
+    // past the end, which must stay representable to read as zeros)
+    if (((int64_t)d->seq_q + 128) * d->q_stride_s * 2 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
     ColArgs a;
     a.q = (const half_t*)q; a.k = (const half_t*)k; a.lse = lse; a.noise = noise;
     a.out_sum = out_sum; a.out_sumsq = out_sumsq;

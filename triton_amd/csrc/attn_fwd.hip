@@ -416,7 +416,7 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
         if (!(d->tau > 0.f)) return TRN_E_UNSUPPORTED;
         if (d->noise_stride_s < d->seq_kv) return TRN_E_STRIDE;
         // one head's noise is addressed with 32-bit byte offsets
-        if ((int64_t)d->seq_q * d->noise_stride_s * 4 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
+        if ((int64_t)d->seq_q * d->noise_stride_s * 4 + 1024 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
         if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
             !pitch16(d->noise_stride_b, 4))
             return TRN_E_ALIGN;
@@ -436,7 +436,8 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
-    if (((int64_t)d->seq_kv + 128) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 128) * d->v_stride_s * 2 > 0x7fffffffLL)
+    // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
+    if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)
         return TRN_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;

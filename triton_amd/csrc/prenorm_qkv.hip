@@ -229,7 +229,8 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     const int64_t pitches[] = {ldx, ldwq, ldwk, ldwv, q_stride_h, q_stride_s, k_stride_h, k_stride_s, v_stride_h, v_stride_s};
     for (int64_t p : pitches) if (!pitch16(p, 2)) return TRN_E_ALIGN;     // 16-byte loads and stores
     // X and W tiles are fetched with 32-bit buffer offsets
-    const int64_t spans[] = {(tokens + GBM) * ldx * 2, (hidden + GBK) * ldwq * 2, (hidden + GBK) * ldwk * 2, (hidden + GBK) * ldwv * 2};
+    // (with room for the tiles the pipelines request past the end, which must stay representable to read as zeros)
+    const int64_t spans[] = {(tokens + 256) * ldx * 2, (hidden + 512) * ldwq * 2, (hidden + 512) * ldwk * 2, (hidden + 512) * ldwv * 2};
     for (int64_t sp : spans) if (sp > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
 
     GemmArgs a;
