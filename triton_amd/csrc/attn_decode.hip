@@ -136,10 +136,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
                 s[r] = (key < a.Skv && (!a.causal || key <= qrow + off)) ? s[r] : -INFINITY;
             }
         }
-        float smax = s[0];
-#pragma unroll
-        for (int r = 1; r < 16; ++r) smax = fmaxf(smax, s[r]);
-        smax = half_max(smax) * a.c1;
+        const float smax = half_max(max16(s)) * a.c1;
         const float mnew = fmaxf(m, smax);
         const float mref = mnew == -INFINITY ? 0.f : mnew;     // a row can see nothing of a block
         const float alpha = fast_exp2(m - mref);               // m = -inf: 0

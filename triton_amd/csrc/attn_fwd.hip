@@ -194,10 +194,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
                 sx[r] = ok ? sx[r] : -INFINITY;      // (a select: stale-LDS garbage past the last block never propagates)
             }
         }
-        smax = sx[0];
-#pragma unroll
-        for (int r = 1; r < 16; ++r) smax = fmaxf(smax, sx[r]);
-        smax = half_max(smax) * a.c1;
+        smax = half_max(max16(sx)) * a.c1;
         return __builtin_amdgcn_ballot_w64(smax > m + 8.0f) != 0;
     };
     auto rescale = [&](float smax) __attribute__((always_inline)) {

@@ -49,6 +49,14 @@ __device__ __forceinline__ half4_t lds_read_tr16(const half_t* p) {
     return __builtin_bit_cast(half4_t, r);
 }
 
+// max of 16 values in 8 three-input maxima (v_max3_f32) instead of a chain of 15 two-input ones
+__device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+__device__ __forceinline__ float max16(const float16_t& s) {
+    const float a = max3(s[0], s[1], s[2]), b = max3(s[3], s[4], s[5]), c = max3(s[6], s[7], s[8]);
+    const float d = max3(s[9], s[10], s[11]), e = max3(s[12], s[13], s[14]);
+    return fmaxf(max3(a, b, s[15]), max3(c, d, e));
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }

@@ -20,7 +20,7 @@
 
 namespace trn {
 
-constexpr int GBM = 128, GBN = 128, GBK = 64;
+[[maybe_unused]] constexpr int GBM = 128, GBN = 128, GBK = 64;
 
 __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
