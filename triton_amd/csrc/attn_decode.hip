@@ -15,7 +15,7 @@ namespace trn {
 
 constexpr int DNW = 8;    // waves per workgroup
 
-template <int D>
+template <int D, bool NOISE>
 __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
     constexpr int NS = D / 16;    // k-steps of S^T = K Q^T; also (2 key halves) x (D/32) MFMAs of P V
@@ -27,7 +27,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     // outstanding global->LDS loads that may alias them, and only distinct variables are provably disjoint
     __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * D];
     __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * D];
-    __shared__ float st_m[DNW][32], st_l[DNW][32];
+    __shared__ float st_m[DNW][32], st_l[DNW][32], st_m2[DNW][32], st_l2[DNW][32];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,21 +112,37 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m = -INFINITY, l = 0.f;       // running max (log2 domain, shared by the lane pair) and this lane's partial sum
+    float m2 = -INFINITY, l2 = 0.f;     // the same for the perturbed scores (KeyFormer)
+    // KeyFormer noise: this lane's query row, the 4 x 4 keys of its accumulator layout per block, one block ahead
+    const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(NOISE ? a.noise + b * a.nb + head * a.nh : nullptr), 0,
+        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
+    const int nvo = NOISE ? (int)(((int64_t)qrow_ld * a.ns + 4 * h) * 4) : 0;
+    float4_t g0[4], g1[4];
+    auto fetch_noise = [&](int blk, float4_t (&g)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            g[r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(nrs, nvo + r4 * 32, blk * 128, 0));
+    };
 
     const int nblk = (a.Skv + 31) / 32;
     const int nmine = (nblk - wave + DNW - 1) / DNW;          // blocks wave, wave + 8, ...
     half8_t ka0[NS], ka1[NS];
 
     // One 32-key block whose K is in kc and whose V is in stage Vc; the next block's loads go to kn / Vn first.
-    auto block = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
+    auto block = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], const half_t* Vc, half_t* Vn, float4_t (&gc)[4],
+                     float4_t (&gn)[4]) __attribute__((always_inline)) {
         const int blk = wave + it * DNW, key0 = blk * 32;
-        fetch_k(blk + DNW, kn);
+        // (with noise the registers are short: K is then single-buffered, refilled as soon as the scores are issued)
+        if constexpr (!NOISE) fetch_k(blk + DNW, kn);
         TRN_FETCH_V(blk + DNW, Vn);
+        if constexpr (NOISE) fetch_noise(blk + DNW, gn);
         float16_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < NS; ++ks) s = mfma32(kc[ks], qB[ks], s);
+        if constexpr (NOISE) fetch_k(blk + DNW, kc);
         // mask (wave-uniform test), block max, running max, probabilities
         const bool masked = (key0 + 32 > a.Skv) || (a.causal && key0 + 31 > off);
         if (masked) {
@@ -134,6 +150,19 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             for (int r = 0; r < 16; ++r) {
                 const int key = key0 + 8 * (r / 4) + 4 * h + (r % 4);
                 s[r] = (key < a.Skv && (!a.causal || key <= qrow + off)) ? s[r] : -INFINITY;
+            }
+        }
+        if constexpr (NOISE) {          // row normaliser of z = (scale*s + g)/tau in the log2 domain (masked: -inf stays -inf)
+            float16_t z;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) z[r] = __builtin_fmaf(gc[r / 4][r % 4], a.c3, s[r] * a.c2);
+            const float zmax = fmaxf(m2, half_max(max16(z)));
+            if (zmax > -INFINITY) {
+                float sum = 0.f;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sum += fast_exp2(z[r] - zmax);
+                l2 = l2 * fast_exp2(m2 - zmax) + sum;
+                m2 = zmax;
             }
         }
         const float smax = half_max(max16(s)) * a.c1;
@@ -155,8 +184,9 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
             for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
         m = mnew;
-        // this block's V has landed: behind it only the next block's NS + NI requests were issued
-        __builtin_amdgcn_s_waitcnt(0x0f70 | ((NS + NI) & 15) | (((NS + NI) >> 4) << 14));
+        // this block's V has landed: behind it only the next block's NS + NI (+ 4 noise) requests were issued
+        constexpr int kBehind = NS + NI + (NOISE ? 4 : 0);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (kBehind & 15) | ((kBehind >> 4) << 14));
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const half_t* vp = Vc + 16 * (i / NDB) * D;
@@ -168,9 +198,15 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     };
     fetch_k(wave, ka0);
     TRN_FETCH_V(wave, Vs0);
+    if constexpr (NOISE) fetch_noise(wave, g0);
     for (int it = 0; it < nmine; it += 2) {
-        block(it, ka0, ka1, Vs0, Vs1);
-        if (it + 1 < nmine) block(it + 1, ka1, ka0, Vs1, Vs0);
+        if constexpr (NOISE) {
+            block(it, ka0, ka0, Vs0, Vs1, g0, g1);
+            if (it + 1 < nmine) block(it + 1, ka0, ka0, Vs1, Vs0, g1, g0);
+        } else {
+            block(it, ka0, ka1, Vs0, Vs1, g0, g1);
+            if (it + 1 < nmine) block(it + 1, ka1, ka0, Vs1, Vs0, g1, g0);
+        }
     }
 #undef TRN_FETCH_V
 
@@ -179,6 +215,10 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     l = half_sum(l);
     __builtin_amdgcn_s_waitcnt(0x0f70);                 // the look-ahead requests past the end have landed too
     if (h == 0) { st_m[wave][c] = m; st_l[wave][c] = l; }
+    if constexpr (NOISE) {
+        l2 = half_sum(l2);
+        if (h == 0) { st_m2[wave][c] = m2; st_l2[wave][c] = l2; }
+    }
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
         float4_t* part = reinterpret_cast<float4_t*>((db < NDB / 2 ? Vs0 : Vs1) + wave * 32 * D);
@@ -215,6 +255,17 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             }
         }
         if (dg == 0 && q < a.Sq && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
+        if constexpr (NOISE) {
+            if (dg == 1 && q < a.Sq) {
+                float ms = st_m2[0][q];
+#pragma unroll
+                for (int w = 1; w < DNW; ++w) ms = fmaxf(ms, st_m2[w][q]);
+                float L2 = 0.f;
+#pragma unroll
+                for (int w = 0; w < DNW; ++w) L2 += st_l2[w][q] * fast_exp2(st_m2[w][q] - ms);
+                a.lse_pert[((int64_t)b * a.Hq + head) * a.Sq + q] = (ms + fast_log2(L2)) * kLn2;
+            }
+        }
     }
 #endif
 }
@@ -222,8 +273,14 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 hipError_t launch_attn_decode(const AttnArgs& a, int head_dim, hipStream_t stream) {
     const int64_t grid = (int64_t)a.B * a.Hq;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    if (head_dim == 128) hipLaunchKernelGGL(attn_decode_kernel<128>, dim3((unsigned)grid), dim3(DNW * 64), 0, stream, a);
-    else hipLaunchKernelGGL(attn_decode_kernel<64>, dim3((unsigned)grid), dim3(DNW * 64), 0, stream, a);
+    const dim3 g((unsigned)grid), t(DNW * 64);
+    if (a.noise) {
+        if (head_dim == 128) hipLaunchKernelGGL((attn_decode_kernel<128, true>), g, t, 0, stream, a);
+        else hipLaunchKernelGGL((attn_decode_kernel<64, true>), g, t, 0, stream, a);
+    } else {
+        if (head_dim == 128) hipLaunchKernelGGL((attn_decode_kernel<128, false>), g, t, 0, stream, a);
+        else hipLaunchKernelGGL((attn_decode_kernel<64, false>), g, t, 0, stream, a);
+    }
     return hipGetLastError();
 }
 

@@ -439,7 +439,7 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
     // a handful of queries per head (decode): one workgroup per head, its waves split the keys
-    if (!noise && d->seq_q <= 32) return launch_attn_decode(a, d->head_dim, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+    if (d->seq_q <= 32) return launch_attn_decode(a, d->head_dim, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
     // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
     // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
     // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to
