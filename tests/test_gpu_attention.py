@@ -41,6 +41,12 @@ CASES = [
     (2, 32, 8, 1024, 1024, 128, True),   # enough workgroups for the 8-wave (256-query) tile shape
     (2, 32, 8, 1000, 1000, 128, False),  # the same, ragged
     (1, 72, 1, 1100, 1100, 64, True),
+    # at most 32 queries per head: the decode kernel (waves split the keys), GQA / MQA, ragged key counts
+    (2, 8, 2, 16, 1040, 128, True),
+    (1, 6, 1, 7, 333, 64, True),
+    (1, 4, 2, 32, 32, 128, True),
+    (3, 4, 4, 32, 5000, 128, False),
+    (1, 4, 2, 33, 1040, 128, True),      # one query more: back to the prefill kernel
 ]
 
 
