@@ -12,8 +12,8 @@
 // and each lane accumulates its 16 per-key partial sums in registers across all query tiles; the sum over
 // the 32 queries held by different lanes is done once at the end.  No atomics: results are deterministic.
 //
-// Q tiles of 64 queries go straight from global memory into two alternating LDS stages (buffer_load ... lds,
-// XOR-swizzled rows), one barrier per tile.  What the VALU needs per tile besides the scores -- the row
+// Q tiles of 64 queries go straight from global memory into a ring of three LDS stages (buffer_load ... lds,
+// XOR-swizzled rows), requested two tiles ahead, one barrier per tile.  What the VALU needs per tile besides the scores -- the row
 // normalisers and, for KeyFormer, the wave's 64 x 32 block of fp32 noise, which is the HBM stream that bounds
 // that variant -- is loaded into registers one whole tile ahead, so that a CU always has about 64 KB of noise
 // in flight.  All of these loads are buffer loads with out-of-range zero fill and are issued unconditionally
@@ -47,6 +47,7 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
     constexpr int NI = CBM / (RPI * 4);        // such loads per wave per stage
     __shared__ __attribute__((aligned(1024))) half_t Qs0[CBM * D];
     __shared__ __attribute__((aligned(1024))) half_t Qs1[CBM * D];
+    __shared__ __attribute__((aligned(1024))) half_t Qs2[CBM * D];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
         NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
     const int nvo = NOISE ? (int)((c * a.ns + wkey0 + 4 * h) * 4) : 0;   // lane's query row, first 4 keys of its 16
     struct Pre { float lse[2]; float4_t g[2][4]; };
-    Pre pre0, pre1;
+    Pre pc, pn;      // this tile's values and the next one's
     auto prefetch = [&](int t, Pre& p) __attribute__((always_inline)) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb)
@@ -167,30 +168,35 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
     };
     // tile t: its stage has landed once this wave's own share has (everything issued behind it is the
     // prefetch of the same tile: 2 normaliser loads and, with noise, 8 noise loads) and the others' too
-    auto tile = [&](int t, const half_t* Qc, half_t* Qn, const Pre& pc, Pre& pn) __attribute__((always_inline)) {
-        if constexpr (NOISE) __builtin_amdgcn_s_waitcnt(0x0f7a); else __builtin_amdgcn_s_waitcnt(0x0f72);
+    // Tile t reads stage t % 3; the stage of tile t+2 is requested as soon as the barrier shows that everybody has
+    // left tile t-1 (its previous tenant), so a Q stage has two tile times to arrive from L2.  Behind this wave's
+    // share of stage t only the register prefetch of tile t and stage t+1 have been issued: NI + 2 (+ 8 with noise)
+    // requests.  All of them are issued unconditionally (past the last tile everything reads as zeros into a stage
+    // nobody uses): the compiler sizes its own waits for prefetched registers by the loads it KNOWS follow them, and
+    // a conditional load counts as absent, which would make every use of a prefetched value drain the refills too.
+    auto tile = [&](int t, const half_t* Qc, half_t* Qf) __attribute__((always_inline)) {
+        constexpr int kBehind = NI + 2 + (NOISE ? 8 : 0);
+        __builtin_amdgcn_s_waitcnt(0x0f70 | (kBehind & 15) | ((kBehind >> 4) << 14));
         __builtin_amdgcn_s_barrier();        // (a bare barrier: nothing else in flight needs draining)
         __builtin_amdgcn_sched_barrier(0);
-        // unconditional (past the last tile everything reads as zeros into a stage nobody uses): the compiler sizes
-        // its waits for the prefetched registers by the loads it KNOWS follow them, and a conditional load counts
-        // as absent, which would make every use of a prefetched value drain the stage refill as well
-        TRN_FETCH_Q(t + 1, Qn);
         prefetch(t + 1, pn);
+        TRN_FETCH_Q(t + 2, Qf);
         __builtin_amdgcn_sched_barrier(0);
         blocks(Qc, t * CBM, pc);
+        pc = pn;                             // (waits for the register prefetch only: the stage request is behind it)
     };
-    if (t0 < nt) {
-        TRN_FETCH_Q(t0, Qs0);
-        prefetch(t0, pre0);
-    }
+    TRN_FETCH_Q(t0, Qs0);
+    prefetch(t0, pc);
+    TRN_FETCH_Q(t0 + 1, Qs1);
     // Pin the arrival of the K rows here, ahead of the loop.  Left to the first MFMA that reads them, the wait the
     // compiler inserts sits inside the loop body and, being conservative across the back edge, drains the stage and
     // prefetch loads of every iteration.
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) asm volatile("" ::"v"(kA[ks]));
-    for (int t = t0; t < nt; t += 2) {
-        tile(t, Qs0, Qs1, pre0, pre1);
-        if (t + 1 < nt) tile(t + 1, Qs1, Qs0, pre1, pre0);
+    for (int t = t0; t < nt; t += 3) {
+        tile(t, Qs0, Qs2);
+        if (t + 1 < nt) tile(t + 1, Qs1, Qs0);
+        if (t + 2 < nt) tile(t + 2, Qs2, Qs1);
     }
 #undef TRN_FETCH_Q
 
