@@ -1,0 +1,148 @@
+"""Counterpart of the reference's benchmark drivers for the hand-written modules.
+
+The reference's `<variant>_<model>_benchmark.py` scripts read IR candidates, generate a module per candidate and time
+its `forward` (vanilla_llama_benchmark.py:131-139 tensors, :243-294 timing, :515-547 result records).  With the code
+generator bypassed there is one candidate per variant -- the hand-written module -- so this driver keeps everything
+either side of it: the tensor configurations (a JSON list of {"M","N","D","H","P"} as in the reference's
+`evaluation/<model>_configs.json`, or the built-in decode shapes), the tensor recipe (`randn.clamp(-1,1)*0.01`, outputs
+zeroed), the timing sequence (cold call, 10 warm-ups on a side stream, capture, 100 graph replays, mean ms) and the
+result records (`ir_id`, `ir_expression`, `execution_time_ms`, `tensor_config`, `error`), appended to `--output`
+one configuration at a time like the reference's incremental save.
+
+    python -m triton_amd.benchmark --variant vanilla --model llama --output vanilla_llama.json
+    python -m triton_amd.benchmark --variant roco --configs my_shapes.json
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+from typing import Dict, List
+
+VARIANTS = ("vanilla", "prenorm", "qknorm", "keyformer", "roco")
+
+
+def tensor_shapes(cfg: Dict[str, int]) -> Dict[str, tuple]:
+    """Shapes of the tensors the reference drivers allocate for a configuration
+    (vanilla_llama_benchmark.py:42-77, keyformer_llama_benchmark.py:74-79, roco_llama_benchmark.py:74-75)."""
+    M, N, D, P = cfg["M"], cfg["N"], cfg["D"], cfg["P"]
+    H = cfg.get("H", N // D)
+    return {"X": (M, N), "WQ": (N, N), "WK": (N, N), "WV": (N, N), "K_cache": (H, P + M, D), "V_cache": (H, P + M, D),
+            "O2": (M, N), "noise": (H, M, P + M), "C_out": (H, P + M), "C_out1": (H, P + M), "C_out2": (H, P + M)}
+
+
+OUTPUTS = ("O2", "C_out", "C_out1", "C_out2")
+
+
+def make_tensors(cfg: Dict[str, int], names: List[str], device: str = "cuda"):
+    """Inputs `randn.clamp(-1, 1) * 0.01`, outputs zero, all fp16 (vanilla_llama_benchmark.py:131-139)."""
+    import torch
+    shapes = tensor_shapes(cfg)
+    out = {}
+    for n in names:
+        if n not in shapes:
+            raise ValueError(f"Unknown tensor parameter: {n}")
+        if n in OUTPUTS:
+            out[n] = torch.zeros(shapes[n], dtype=torch.float16, device=device)
+        else:
+            out[n] = torch.randn(shapes[n], dtype=torch.float16, device=device).clamp(-1, 1) * 0.01
+    return out
+
+
+def time_module(module, tensors, warmup_runs: int = 10, benchmark_runs: int = 100) -> float:
+    """Mean milliseconds per `forward`, measured as the reference does (vanilla_llama_benchmark.py:243-294)."""
+    import torch
+    for n in OUTPUTS:
+        if n in tensors:
+            tensors[n].zero_()
+    args = [tensors[p] for p in module.TENSOR_PARAMS]
+    stream = torch.cuda.Stream()
+    module.forward(*args)                       # first call (the reference's autotune call)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        for _ in range(warmup_runs):
+            module.forward(*args)
+    stream.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            module.forward(*args)
+    stream.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    with torch.cuda.stream(stream):
+        start.record()
+        for _ in range(benchmark_runs):
+            graph.replay()
+        end.record()
+    stream.synchronize()
+    if "O2" in tensors and torch.isnan(tensors["O2"]).any().item():
+        print(f"WARNING: NaN values detected in O2 tensor!")
+    return start.elapsed_time(end) / benchmark_runs
+
+
+def append_record(path: str, record: dict) -> None:
+    """The reference's incremental save: read the list, append, write back (vanilla_llama_benchmark.py:515-547)."""
+    try:
+        with open(path) as f:
+            data = json.load(f)
+    except (OSError, ValueError):
+        data = []
+    data.append(record)
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    with open(path, "w") as f:
+        json.dump(data, f, indent=2)
+
+
+def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: int = 10, benchmark_runs: int = 100) -> List[dict]:
+    import torch
+
+    from . import modules
+    if not torch.cuda.is_available():
+        raise SystemExit("Error: no GPU available; the hand-written kernels have no CPU path")
+    records = []
+    for cfg in configs:
+        rec = {"ir_id": f"trinity_hip/{variant}", "ir_expression": f"hand-written gfx950 module ({variant}, decode-append form)",
+               "execution_time_ms": float("inf"), "tensor_config": dict(cfg), "error": None}
+        try:
+            consts = {"head_dim": cfg["D"]}
+            module = modules.get(variant, "decode", **consts)
+            tensors = make_tensors(cfg, module.TENSOR_PARAMS)
+            rec["execution_time_ms"] = time_module(module, tensors, warmup_runs, benchmark_runs)
+        except Exception as e:          # the reference records a failing candidate and carries on (:329-332)
+            rec["error"] = str(e)
+        records.append(rec)
+        append_record(output, rec)
+        print(f"  {rec['ir_id']} {rec['tensor_config']}: "
+              + (f"{rec['execution_time_ms']:.4f} ms" if rec["error"] is None else f"error: {rec['error']}"))
+        torch.cuda.empty_cache()
+    return records
+
+
+def main(argv=None) -> int:
+    from . import configs as shapes
+    ap = argparse.ArgumentParser(description="Time the hand-written module of one variant the way the reference's drivers time a candidate")
+    ap.add_argument("--variant", choices=VARIANTS, default="vanilla")
+    ap.add_argument("--model", choices=("llama", "falcon"), default="llama",
+                    help="built-in decode shape (M=16, P=1024 at the model's widths) when --configs is not given")
+    ap.add_argument("--configs", type=str, default=None, help="JSON file: a list of {M, N, D, H, P} tensor configurations")
+    ap.add_argument("--output", type=str, default=None, help="result file (default ./<variant>_<model>.json)")
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--runs", type=int, default=100)
+    a = ap.parse_args(argv)
+    if a.configs:
+        with open(a.configs) as f:
+            cfgs = json.load(f)
+        if not isinstance(cfgs, list) or not all(isinstance(c, dict) and {"M", "N", "D", "P"} <= set(c) for c in cfgs):
+            ap.error("--configs: expected a JSON list of objects with M, N, D, P (and optionally H)")
+    else:
+        cfgs = [dict(shapes.DECODE_LLAMA if a.model == "llama" else shapes.DECODE_FALCON)]
+    out = a.output or f"./{a.variant}_{a.model}.json"
+    with open(out, "w") as f:               # the reference starts a run from an empty list (:476)
+        json.dump([], f)
+    run(a.variant, cfgs, out, a.warmup, a.runs)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
