@@ -2,7 +2,7 @@
 summary: per-kernel call counts and average durations (`--kernel-trace --stats` runs) and per-kernel
 counter values averaged per dispatch (`--pmc` runs).
 
-    python -m triton_amd.profiling gpurun_out/prof/attn_results.db [--filter trn::] [--calib-bytes N]
+    python -m triton_amd.profiling /tmp/prof/attn_results.db [--filter trn::] [--calib-bytes N]
 
 With --calib-bytes N the FETCH_SIZE / WRITE_SIZE readings (KiB per dispatch) of every kernel are also
 shown scaled by what the library's calibration copy kernel read for its known N bytes.
