@@ -37,6 +37,7 @@ def parse():
     ap.add_argument("--workload", default="default",
                     help="default (vanilla headline + rmsnorm), all, or one of vanilla rmsnorm prenorm qknorm keyformer roco decode")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="with --workload all: skip the decode-append timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain copy kernel on 256 MiB (3 launches) so that a rocprofv3 --pmc run "
@@ -306,7 +307,7 @@ def main():
         if wl in ("all", name):
             extra[name] = bench_variant(name, max(a.steps // 4, 10), a.warmup)
             torch.cuda.empty_cache()
-    if wl in ("all", "decode"):
+    if wl == "decode" or (wl == "all" and not a.no_decode):
         extra["decode_append_M16_P1024"] = bench_decode(100, a.warmup)
     if van is None:                       # a single non-headline workload was asked for
         print(json.dumps({"workload": wl, **extra}))
