@@ -107,6 +107,23 @@ int trn_attn_fwd_f16(const trn_attn_desc* desc, const void* q, const void* k, co
                      const float* noise, float* lse_pert, void* stream);
 
 /*
+ * trn_attn_fwd_f16 with a caller-provided workspace.  In the reference every cross-kernel intermediate is a
+ * caller-allocated tensor passed to `forward` (C, C_exp, C_sum ... in vanilla_llama_benchmark.py:42-77, zero-filled
+ * by the driver, :237-240); this is that convention for the one intermediate these kernels have.  For decode shapes
+ * (seq_q <= 32) with few heads the keys are then split over several workgroups per head, whose partial results and
+ * arrival counters live in the workspace; for every other shape, or with workspace == NULL or too small, the call is
+ * exactly trn_attn_fwd_f16.
+ *   workspace        device memory, 256-byte aligned, trn_attn_workspace_bytes(desc) bytes, zero-filled ONCE before
+ *                    its first use (the kernel returns its counters to zero).  One call at a time may use it.
+ * trn_attn_workspace_bytes returns 0 when the shape would not use a workspace.
+ */
+int64_t trn_attn_workspace_bytes(const trn_attn_desc* desc);
+int trn_attn_fwd_ws_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                        void* o, float* lse, const void* gamma_q,
+                        const float* noise, float* lse_pert,
+                        void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * Per-key column statistics of the attention probabilities, given the row normalisers from
  * trn_attn_fwd_f16:   p_ij = exp(t_ij - lse_i),  out_sum[j] = sum_i p_ij,
  * out_sumsq[j] = sum_i p_ij^2, over the queries i that can see key j.

@@ -13,9 +13,14 @@ struct AttnArgs {
     float c2, c3;  // scale*log2(e)/tau, log2(e)/tau     : perturbed scores  z2 = s*c2 + g*c3
     float q_eps;
     int causal, q_norm;
+    // decode kernel only: keys split over n_split workgroups per head, partial results and arrival counters in ws
+    int n_split;
+    float* ws;
 };
 
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).
-hipError_t launch_attn_decode(const AttnArgs& a, int head_dim, hipStream_t stream);
+hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+// Bytes of workspace with which launch_attn_decode splits the keys of this problem over several workgroups (0: it would not).
+int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq_kv, int head_dim);
 
 }  // namespace trn

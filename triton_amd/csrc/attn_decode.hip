@@ -11,6 +11,11 @@
 // that the waits can be counted.
 #include "attn.h"
 
+#ifndef TRN_ARRIVAL_ORDER
+#define TRN_ARRIVAL_ORDER __ATOMIC_RELAXED
+#endif
+typedef unsigned long long ulong2_t __attribute__((ext_vector_type(2)));
+
 namespace trn {
 
 constexpr int DNW = 8;    // waves per workgroup
@@ -31,7 +36,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int j = blockIdx.x;
+    const int j = blockIdx.x / a.n_split, split = blockIdx.x % a.n_split;
     const int G = a.Hq / a.Hkv, nkv = a.B * a.Hkv;
     const int kvslot = j % nkv, g = j / nkv;
     const int b = kvslot / a.Hkv, kvh = kvslot % a.Hkv, head = kvh * G + g;
@@ -45,31 +50,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * h;
 #pragma unroll
         for (int ks = 0; ks < NS; ++ks) qB[ks] = *reinterpret_cast<const half8_t*>(qp + ks * 16);
-        if (a.q_norm) {
-            float ss = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < NS; ++ks)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) { float f = (float)qB[ks][e]; ss += f * f; }
-            ss = half_sum(ss);
-            const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
-#pragma unroll
-            for (int ks = 0; ks < NS; ++ks) {
-                half8_t gq;
-                if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 16 + 8 * h);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float y = (float)qB[ks][e] * rstd;
-                    if (a.gamma_q) y = (float)gq[e] * y;
-                    qB[ks][e] = (half_t)y;
-                }
-            }
-        }
     }
-    // pin the arrival of Q here: left to the first MFMA in the loop, the compiler's wait would sit in the loop body
-#pragma unroll
-    for (int ks = 0; ks < NS; ++ks) asm volatile("" ::"v"(qB[ks]));
-
     // ---- K: block rows straight into registers as A operands (lane: key c of the block, columns ks*16 + 8h ..)
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.k + b * a.kb + kvh * a.kh), 0, (int)(((int64_t)(a.Skv - 1) * a.ks + D) * 2), 0x00020000);
@@ -125,14 +106,16 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             g[r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(nrs, nvo + r4 * 32, blk * 128, 0));
     };
 
-    const int nblk = (a.Skv + 31) / 32;
-    const int nmine = (nblk - wave + DNW - 1) / DNW;          // blocks wave, wave + 8, ...
+    // this workgroup's blocks: a contiguous share of the keys when they are split over several workgroups
+    const int nblk_all = (a.Skv + 31) / 32, bps = (nblk_all + a.n_split - 1) / a.n_split;
+    const int blk0 = split * bps, nblk = max(0, min(nblk_all, blk0 + bps) - blk0);
+    const int nmine = nblk > wave ? (nblk - wave + DNW - 1) / DNW : 0;          // blocks blk0 + wave, + 8, ...
     half8_t ka0[NS], ka1[NS];
 
     // One 32-key block whose K is in kc and whose V is in stage Vc; the next block's loads go to kn / Vn first.
     auto block = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], const half_t* Vc, half_t* Vn, float4_t (&gc)[4],
                      float4_t (&gn)[4]) __attribute__((always_inline)) {
-        const int blk = wave + it * DNW, key0 = blk * 32;
+        const int blk = blk0 + wave + it * DNW, key0 = blk * 32;
         // (with noise the registers are short: K is then single-buffered, refilled as soon as the scores are issued)
         if constexpr (!NOISE) fetch_k(blk + DNW, kn);
         TRN_FETCH_V(blk + DNW, Vn);
@@ -196,9 +179,33 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             oacc[i % NDB] = mfma32(va, pB[i / NDB], oacc[i % NDB]);
         }
     };
-    fetch_k(wave, ka0);
-    TRN_FETCH_V(wave, Vs0);
-    if constexpr (NOISE) fetch_noise(wave, g0);
+    fetch_k(blk0 + wave, ka0);
+    TRN_FETCH_V(blk0 + wave, Vs0);
+    if constexpr (NOISE) fetch_noise(blk0 + wave, g0);
+    // (the first K / V requests are on their way before Q is waited for: one memory latency instead of two)
+    if (a.q_norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < NS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { float f = (float)qB[ks][e]; ss += f * f; }
+        ss = half_sum(ss);
+        const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
+#pragma unroll
+        for (int ks = 0; ks < NS; ++ks) {
+            half8_t gq;
+            if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 16 + 8 * h);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                float y = (float)qB[ks][e] * rstd;
+                if (a.gamma_q) y = (float)gq[e] * y;
+                qB[ks][e] = (half_t)y;
+            }
+        }
+    }
+    // pin the arrival of Q here: left to the first MFMA in the loop, the compiler's wait would sit in the loop body
+#pragma unroll
+    for (int ks = 0; ks < NS; ++ks) asm volatile("" ::"v"(qB[ks]));
     for (int it = 0; it < nmine; it += 2) {
         if constexpr (NOISE) {
             block(it, ka0, ka0, Vs0, Vs1, g0, g1);
@@ -228,50 +235,154 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
                 float4_t{oacc[db][r4 * 4], oacc[db][r4 * 4 + 1], oacc[db][r4 * 4 + 2], oacc[db][r4 * 4 + 3]};
     }
     __syncthreads();
+    const int q = tid & 31, dg = tid >> 5;                // 16 groups of threads share out the D/4 quads of a query
+    constexpr int NQD = (D / 4) / 16;                     // quads per thread
+    float mstar = st_m[0][q];
+#pragma unroll
+    for (int w = 1; w < DNW; ++w) mstar = fmaxf(mstar, st_m[w][q]);
+    float L = 0.f;
+    float4_t acc[NQD];
     {
-        const int q = tid & 31, dg = tid >> 5;            // 16 groups of threads share out the D/4 quads of a query
-        float mstar = st_m[0][q];
+        float wgt[DNW];
 #pragma unroll
-        for (int w = 1; w < DNW; ++w) mstar = fmaxf(mstar, st_m[w][q]);
-        float wgt[DNW], L = 0.f;
+        for (int w = 0; w < DNW; ++w) {                   // idle waves: m = -inf, weight 0
+            wgt[w] = mstar == -INFINITY ? 0.f : fast_exp2(st_m[w][q] - mstar);
+            L += st_l[w][q] * wgt[w];
+        }
 #pragma unroll
-        for (int w = 0; w < DNW; ++w) { wgt[w] = fast_exp2(st_m[w][q] - mstar); L += st_l[w][q] * wgt[w]; }   // idle waves: m = -inf, weight 0
-        const float inv = 1.0f / L;
-        half_t* orow = a.o + b * a.ob + head * a.oh + (int64_t)q * a.os;
-#pragma unroll
-        for (int qi = 0; qi < (D / 4) / 16; ++qi) {
+        for (int qi = 0; qi < NQD; ++qi) {
             const int quad = dg + 16 * qi;                // d = 4*quad .. +3
             const half_t* base = quad < D / 8 ? Vs0 : Vs1;
             const int ql = quad % (D / 8);
-            float4_t acc = {0.f, 0.f, 0.f, 0.f};
+            acc[qi] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int w = 0; w < DNW; ++w) {
-                const float4_t v = reinterpret_cast<const float4_t*>(base + w * 32 * D)[ql * 32 + q];
-                acc += v * wgt[w];
+            for (int w = 0; w < DNW; ++w) acc[qi] += reinterpret_cast<const float4_t*>(base + w * 32 * D)[ql * 32 + q] * wgt[w];
+        }
+    }
+    float ms2 = -INFINITY, L2 = 0.f;
+    if constexpr (NOISE) {
+#pragma unroll
+        for (int w = 0; w < DNW; ++w) ms2 = fmaxf(ms2, st_m2[w][q]);
+#pragma unroll
+        for (int w = 0; w < DNW; ++w) L2 += ms2 == -INFINITY ? 0.f : st_l2[w][q] * fast_exp2(st_m2[w][q] - ms2);
+    }
+    const int bh = b * a.Hq + head;
+    if (a.n_split > 1) {
+        // ---- keys split over workgroups: publish (m, l, unnormalised O) of this share; the workgroup that arrives
+        // last at the head's counter merges all shares.  Workspace: [arrival counters, 256-byte aligned][bh][split]
+        // {O as quads [D/4][32 queries][4], (m, l, m2, l2) [32]} floats.  The shares travel as device-scope atomic stores and loads, which
+        // go to the memory all L2 slices agree on (a fence that makes ordinary stores visible writes back and
+        // invalidates a whole L2, and with one per wave that took several times the kernel's own time); the arrival
+        // is a release/acquire increment by one thread, tied to the other threads by the workgroup barriers.
+        constexpr int PART = 32 * (D + 4);
+        const int n_bh = a.B * a.Hq;
+        unsigned* counters = reinterpret_cast<unsigned*>(a.ws);
+        float* parts = a.ws + ((n_bh + 63) / 64) * 64;
+        float* mine = parts + ((int64_t)bh * a.n_split + split) * PART;
+        auto publish = [](float* p, float4_t v) __attribute__((always_inline)) {
+            const ulong2_t u = __builtin_bit_cast(ulong2_t, v);
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(p), u[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(reinterpret_cast<unsigned long long*>(p) + 1, u[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        };
+        auto collect = [](const float* p) __attribute__((always_inline)) {
+            ulong2_t u;
+            u[0] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u[1] = __hip_atomic_load(reinterpret_cast<const unsigned long long*>(p) + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            return __builtin_bit_cast(float4_t, u);
+        };
+#pragma unroll
+        for (int qi = 0; qi < NQD; ++qi) publish(mine + ((dg + 16 * qi) * 32 + q) * 4, acc[qi]);
+        if (dg == 0) publish(mine + 32 * D + 4 * q, float4_t{mstar, L, ms2, L2});
+        __syncthreads();                                   // every wave's stores have been acknowledged
+        __shared__ unsigned arrival;
+        if (tid == 0) arrival = __hip_atomic_fetch_add(&counters[bh], 1u, TRN_ARRIVAL_ORDER, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (arrival != (unsigned)(a.n_split - 1)) return;
+        const float* head_parts = parts + (int64_t)bh * a.n_split * PART;
+        // shares are fetched eight at a time (all requests of a batch in flight together) and folded in with a
+        // running maximum, in share order: the result does not depend on which workgroup does the merge
+        mstar = -INFINITY; ms2 = -INFINITY; L = 0.f; L2 = 0.f;
+#pragma unroll
+        for (int qi = 0; qi < NQD; ++qi) acc[qi] = float4_t{0.f, 0.f, 0.f, 0.f};
+        constexpr int BATCH = 8;
+        for (int s0 = 0; s0 < a.n_split; s0 += BATCH) {
+            float4_t st[BATCH], d[BATCH][NQD];
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                const float* ps = head_parts + min(s0 + u, a.n_split - 1) * PART;
+                st[u] = collect(ps + 32 * D + 4 * q);
+#pragma unroll
+                for (int qi = 0; qi < NQD; ++qi) d[u][qi] = collect(ps + ((dg + 16 * qi) * 32 + q) * 4);
             }
-            if (q < a.Sq) {
-                const half4_t ov = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv), (half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
-                *reinterpret_cast<half4_t*>(orow + 4 * quad) = ov;
+#pragma unroll
+            for (int u = 0; u < BATCH; ++u) {
+                if (s0 + u >= a.n_split) break;
+                const float mnew = fmaxf(mstar, st[u][0]);
+                if (mnew > -INFINITY) {                        // -inf: a share that saw no key of this query
+                    const float wa = fast_exp2(mstar - mnew), wb = fast_exp2(st[u][0] - mnew);
+                    L = L * wa + st[u][1] * wb;
+#pragma unroll
+                    for (int qi = 0; qi < NQD; ++qi) acc[qi] = acc[qi] * wa + d[u][qi] * wb;
+                    mstar = mnew;
+                }
+                if constexpr (NOISE) {
+                    const float m2new = fmaxf(ms2, st[u][2]);
+                    if (m2new > -INFINITY) {
+                        L2 = L2 * fast_exp2(ms2 - m2new) + st[u][3] * fast_exp2(st[u][2] - m2new);
+                        ms2 = m2new;
+                    }
+                }
             }
         }
-        if (dg == 0 && q < a.Sq && a.lse) a.lse[((int64_t)b * a.Hq + head) * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
-        if constexpr (NOISE) {
-            if (dg == 1 && q < a.Sq) {
-                float ms = st_m2[0][q];
+        if (tid == 0) __hip_atomic_store(&counters[bh], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);                   // left as found: the next launch on the stream starts from zero
+    }
+    {
+        const float inv = 1.0f / L;
+        half_t* orow = a.o + b * a.ob + head * a.oh + (int64_t)q * a.os;
+        if (q < a.Sq) {
 #pragma unroll
-                for (int w = 1; w < DNW; ++w) ms = fmaxf(ms, st_m2[w][q]);
-                float L2 = 0.f;
-#pragma unroll
-                for (int w = 0; w < DNW; ++w) L2 += st_l2[w][q] * fast_exp2(st_m2[w][q] - ms);
-                a.lse_pert[((int64_t)b * a.Hq + head) * a.Sq + q] = (ms + fast_log2(L2)) * kLn2;
+            for (int qi = 0; qi < NQD; ++qi) {
+                const half4_t ov = {(half_t)(acc[qi][0] * inv), (half_t)(acc[qi][1] * inv), (half_t)(acc[qi][2] * inv), (half_t)(acc[qi][3] * inv)};
+                *reinterpret_cast<half4_t*>(orow + 4 * (dg + 16 * qi)) = ov;
             }
+        }
+        if (dg == 0 && q < a.Sq && a.lse) a.lse[(int64_t)bh * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
+        if constexpr (NOISE) {
+            if (dg == 1 && q < a.Sq) a.lse_pert[(int64_t)bh * a.Sq + q] = (ms2 + fast_log2(L2)) * kLn2;
         }
     }
 #endif
 }
 
-hipError_t launch_attn_decode(const AttnArgs& a, int head_dim, hipStream_t stream) {
-    const int64_t grid = (int64_t)a.B * a.Hq;
+// Keys are split over workgroups when one workgroup per head would leave most of the chip idle and a head has enough
+// key blocks to repay the merge: publishing, arriving and collecting cost about 4 us, which is what some 32 blocks of a
+// 128-wide head (twice as many of a 64-wide one) take a single workgroup.  Measured with 16 queries per head, 32 heads
+// of width 128: 1040 keys 14.8 -> 14.5 us, 4112 keys 43 -> 24 us, 16400 keys 154 -> 50 us; 8 heads, 16400 keys
+// 150 -> 26 us.  The caller provides the workspace for the partial results.
+static int decode_splits(int batch, int n_q_heads, int seq_kv, int head_dim) {
+    const int n_bh = batch * n_q_heads, nblk = (seq_kv + 31) / 32;
+    if (n_bh >= 128 || (int64_t)nblk * head_dim < 32 * 128) return 1;
+    const int ns = max(1, min(min(16, 256 / n_bh), nblk / 4));
+    const int bps = (nblk + ns - 1) / ns;                 // blocks per share, as the kernel computes it
+    return (nblk + bps - 1) / bps;                        // no empty share: the last one starts inside the keys
+}
+
+int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq_kv, int head_dim) {
+    if (seq_q > 32) return 0;
+    const int ns = decode_splits(batch, n_q_heads, seq_kv, head_dim);
+    if (ns <= 1) return 0;
+    const int64_t n_bh = (int64_t)batch * n_q_heads;
+    return ((n_bh + 63) / 64) * 256 + n_bh * ns * 32 * (head_dim + 4) * 4;
+}
+
+hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
+    a.n_split = 1; a.ws = nullptr;
+    const int64_t need = attn_decode_workspace_bytes(a.B, a.Hq, a.Sq, a.Skv, head_dim);
+    if (workspace && need > 0 && workspace_bytes >= need) {
+        a.n_split = decode_splits(a.B, a.Hq, a.Skv, head_dim);
+        a.ws = static_cast<float*>(workspace);
+    }
+    const int64_t grid = (int64_t)a.B * a.Hq * a.n_split;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 g((unsigned)grid), t(DNW * 64);
     if (a.noise) {

@@ -399,10 +399,23 @@ int validate_attn(const trn_attn_desc* d, bool need_v) {
 
 }  // namespace trn
 
+extern "C" int64_t trn_attn_workspace_bytes(const trn_attn_desc* d) {
+    using namespace trn;
+    if (!d || validate_attn(d, true) != TRN_OK) return 0;
+    return attn_decode_workspace_bytes(d->batch, d->n_q_heads, d->seq_q, d->seq_kv, d->head_dim);
+}
+
 extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
                                 float* lse, const void* gamma_q, const float* noise, float* lse_pert,
                                 void* stream) {
+    return trn_attn_fwd_ws_f16(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, stream);
+}
+
+extern "C" int trn_attn_fwd_ws_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                   float* lse, const void* gamma_q, const float* noise, float* lse_pert,
+                                   void* workspace, int64_t workspace_bytes, void* stream) {
     using namespace trn;
+    if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;
     if (!d || !q || !k || !v || !o) return TRN_E_NULL;
     if (noise && !lse_pert) return TRN_E_NULL;
     int st = validate_attn(d, true);
@@ -439,7 +452,8 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
     // a handful of queries per head (decode): one workgroup per head, its waves split the keys
-    if (d->seq_q <= 32) return launch_attn_decode(a, d->head_dim, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+    if (d->seq_q <= 32)
+        return launch_attn_decode(a, d->head_dim, workspace, workspace_bytes, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
     // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
     // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
     // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to

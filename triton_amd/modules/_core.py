@@ -261,6 +261,21 @@ class _DecodeAppend(FusedModule):
     def _o_view(O2, H, M, D):
         return O2.view(M, H, D).permute(1, 0, 2).unsqueeze(0)               # [1,H,M,D] view of token-major O2
 
+    def _attend(self, q, K_cache, V_cache, O2, **kw):
+        """Attention of the M new queries over the whole cache, with a workspace (allocated and zeroed once per shape;
+        every call leaves its counters at zero again) so that the keys of a head can be split over several workgroups."""
+        H, M, D = q.shape
+        o = self._o_view(O2, H, M, D)
+        nbytes = ops.attention_workspace_bytes(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal)
+        ws = None
+        if nbytes:
+            key = ("attn_ws", (nbytes,), torch.uint8, str(q.device))
+            fresh = key not in self._ws
+            ws = self._workspace("attn_ws", (nbytes,), torch.uint8, q.device)
+            if fresh:
+                ws.zero_()
+        ops.attention(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal, workspace=ws, **kw)
+
 
 class DecodeVanilla(_DecodeAppend):
     """Vanila.forward / PreNorm.forward (ref_rms.py:45-83 / 101-127)."""
@@ -268,8 +283,7 @@ class DecodeVanilla(_DecodeAppend):
 
     def _run(self, K_cache, O2, V_cache, WK, WQ, WV, X):
         q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
-        H, M, D = q.shape
-        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal)
+        self._attend(q, K_cache, V_cache, O2)
 
 
 class DecodeQKNorm(_DecodeAppend):
@@ -281,8 +295,7 @@ class DecodeQKNorm(_DecodeAppend):
         q, P = self._project(X, WQ, WK, WV, K_cache, V_cache)
         H, M, D = q.shape
         ops.head_rmsnorm(K_cache, None, K_cache, 0.0, row_start=P)          # in place, rows P.. only
-        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
-                      q_norm=True, gamma_q=None, q_eps=0.0)
+        self._attend(q, K_cache, V_cache, O2, q_norm=True, gamma_q=None, q_eps=0.0)
 
 
 class DecodeKeyFormer(_DecodeAppend):
@@ -306,8 +319,7 @@ class DecodeKeyFormer(_DecodeAppend):
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
         score = C_out.view(1, H, PM) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
             self._workspace("score32", (1, H, PM), torch.float32, X.device)
-        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
-                      noise=n4, tau=self.tau, lse_pert=lsep)
+        self._attend(q, K_cache, V_cache, O2, noise=n4, tau=self.tau, lse_pert=lsep)
         ops.attention_colstats(q[None], K_cache[None], lsep, self.scale, self.causal, score, None, noise=n4, tau=self.tau)
         _store_scores(C_out, score)
 
@@ -325,7 +337,7 @@ class DecodeRoCo(_DecodeAppend):
         for i, c in enumerate((C_out1, C_out2)):
             outs.append(c.view(1, H, PM) if c.dtype == torch.float32 and c.is_contiguous() else
                         self._workspace(f"stat32_{i}", (1, H, PM), torch.float32, X.device))
-        ops.attention(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal, lse=lse)
+        self._attend(q, K_cache, V_cache, O2, lse=lse)
         ops.attention_colstats(q[None], K_cache[None], lse, self.scale, self.causal, outs[0], outs[1])
         _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
 

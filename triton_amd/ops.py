@@ -108,9 +108,11 @@ def _row_stat(t: Optional[torch.Tensor], name: str, shape) -> None:
 def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor] = None,
               q_norm: bool = False, gamma_q: Optional[torch.Tensor] = None, q_eps: float = 0.0,
               noise: Optional[torch.Tensor] = None, tau: float = 1.0,
-              lse_pert: Optional[torch.Tensor] = None) -> None:
+              lse_pert: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> None:
     """o = softmax(scale * q k^T [+causal]) v.  q,o [B,Hq,Sq,D]; k,v [B,Hkv,Skv,D] (strided views allowed).
-    Optional outputs: lse [B,Hq,Sq] fp32; with noise [B,Hq,Sq,Skv] fp32 also lse_pert."""
+    Optional outputs: lse [B,Hq,Sq] fp32; with noise [B,Hq,Sq,Skv] fp32 also lse_pert.
+    workspace: optional zero-initialised uint8 tensor of attention_workspace_bytes(...) bytes (decode shapes with
+    few heads then split their keys over several workgroups)."""
     d = _attn_desc(q, k, v, o, scale, causal, q_norm, q_eps, noise, tau)
     B, Hq, Sq, _ = q.shape
     _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq))
@@ -119,9 +121,21 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
         _need(gamma_q.shape == (q.shape[3],), "gamma_q: expected (head_dim,)")
     _need(noise is None or lse_pert is not None, "noise given without lse_pert")
     lib = _lib.load()
+    if workspace is not None:
+        _need(workspace.is_cuda and workspace.is_contiguous() and workspace.dtype == torch.uint8, "workspace: expected a contiguous uint8 GPU tensor")
+        st = lib.trn_attn_fwd_ws_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
+                                     _ptr(noise), _ptr(lse_pert), _ptr(workspace), workspace.numel(), _stream(q))
+        _lib.check("trn_attn_fwd_ws_f16", st)
+        return
     st = lib.trn_attn_fwd_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
                               _ptr(noise), _ptr(lse_pert), _stream(q))
     _lib.check("trn_attn_fwd_f16", st)
+
+
+def attention_workspace_bytes(q, k, v, o, scale: float, causal: bool) -> int:
+    """Bytes of workspace with which `attention` would split the keys of this problem over several workgroups (0: none)."""
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, None, 1.0)
+    return int(_lib.load().trn_attn_workspace_bytes(C.byref(d)))
 
 
 def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
