@@ -11,6 +11,10 @@ one configuration at a time like the reference's incremental save.
 
     python -m triton_amd.benchmark --variant vanilla --model llama --output vanilla_llama.json
     python -m triton_amd.benchmark --variant roco --configs my_shapes.json
+    python -m triton_amd.benchmark --ir candidates.txt --start 0 --num 10      # recognise and time IR candidates
+
+With `--ir` the candidates of an IR file (`id: expression` lines) are each mapped to the module that computes them
+(triton_amd/ir.py) and timed under their own `ir_id`; one that is not an attention variant is recorded with its error.
 """
 from __future__ import annotations
 
@@ -18,7 +22,7 @@ import argparse
 import json
 import os
 import sys
-from typing import Dict, List
+from typing import Dict, List, Optional
 
 VARIANTS = ("vanilla", "prenorm", "qknorm", "keyformer", "roco")
 
@@ -94,29 +98,63 @@ def append_record(path: str, record: dict) -> None:
         json.dump(data, f, indent=2)
 
 
-def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: int = 10, benchmark_runs: int = 100) -> List[dict]:
+def candidates_from_ir(path: str, start: int = 0, num: Optional[int] = 10) -> List[tuple]:
+    """(ir_id, expression, variant or None, reason) for the candidates of an IR file with id >= start, at most `num`
+    of them (the reference's --start / --num / --end, vanilla_llama_benchmark.py:749-753); each is recognised by its
+    dataflow instead of being compiled."""
+    from . import ir
+    out = []
+    for ir_id, expr in ir.read_ir_file(path):
+        if ir_id < start or (num is not None and len(out) >= num):
+            continue
+        m = ir.recognise(expr)
+        out.append((ir_id, expr, m.variant, m.reason))
+    return out
+
+
+def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: int = 10, benchmark_runs: int = 100,
+        candidates: Optional[List[tuple]] = None) -> List[dict]:
     import torch
 
     from . import modules
     if not torch.cuda.is_available():
         raise SystemExit("Error: no GPU available; the hand-written kernels have no CPU path")
+    if candidates is None:              # no IR file: the one candidate is the hand-written module of `variant`
+        candidates = [(f"trinity_hip/{variant}", f"hand-written gfx950 module ({variant}, decode-append form)", variant, "")]
     records = []
     for cfg in configs:
-        rec = {"ir_id": f"trinity_hip/{variant}", "ir_expression": f"hand-written gfx950 module ({variant}, decode-append form)",
-               "execution_time_ms": float("inf"), "tensor_config": dict(cfg), "error": None}
-        try:
-            consts = {"head_dim": cfg["D"]}
-            module = modules.get(variant, "decode", **consts)
-            tensors = make_tensors(cfg, module.TENSOR_PARAMS)
-            rec["execution_time_ms"] = time_module(module, tensors, warmup_runs, benchmark_runs)
-        except Exception as e:          # the reference records a failing candidate and carries on (:329-332)
-            rec["error"] = str(e)
-        records.append(rec)
-        append_record(output, rec)
-        print(f"  {rec['ir_id']} {rec['tensor_config']}: "
-              + (f"{rec['execution_time_ms']:.4f} ms" if rec["error"] is None else f"error: {rec['error']}"))
+        for ir_id, expr, var, reason in candidates:
+            rec = {"ir_id": ir_id, "ir_expression": expr, "execution_time_ms": float("inf"), "tensor_config": dict(cfg), "error": None}
+            try:
+                if var is None:         # the reference records a candidate it cannot compile and carries on (:206-210)
+                    raise ValueError(f"unsupported IR: {reason}")
+                module = modules.get(var, "decode", head_dim=cfg["D"])
+                tensors = make_tensors(cfg, module.TENSOR_PARAMS)
+                rec["execution_time_ms"] = time_module(module, tensors, warmup_runs, benchmark_runs)
+            except Exception as e:      # ... and one that fails at run time (:329-332)
+                rec["error"] = str(e)
+            records.append(rec)
+            append_record(output, rec)
+            print(f"  IR {rec['ir_id']}" + (f" [{var}]" if var else "") + f" {rec['tensor_config']}: "
+                  + (f"{rec['execution_time_ms']:.4f} ms" if rec["error"] is None else f"error: {rec['error']}"))
         torch.cuda.empty_cache()
     return records
+
+
+def print_report(records: List[dict], top_k: int) -> None:
+    """Best candidates per tensor configuration (vanilla_llama_benchmark.py:574-602)."""
+    seen = []
+    for r in records:
+        if r["tensor_config"] not in seen:
+            seen.append(r["tensor_config"])
+    for i, cfg in enumerate(seen):
+        print(f"\nConfiguration {i + 1}:\n  Tensor Shape: M={cfg['M']}, N={cfg['N']}")
+        valid = sorted((r for r in records if r["tensor_config"] == cfg and r["error"] is None),
+                       key=lambda r: r["execution_time_ms"])[:top_k]
+        if not valid:
+            print("  No valid kernels found for this configuration")
+        for j, r in enumerate(valid):
+            print(f"    {j + 1}. IR {r['ir_id']}: {r['execution_time_ms']:.4f} ms")
 
 
 def main(argv=None) -> int:
@@ -127,6 +165,12 @@ def main(argv=None) -> int:
                     help="built-in decode shape (M=16, P=1024 at the model's widths) when --configs is not given")
     ap.add_argument("--configs", type=str, default=None, help="JSON file: a list of {M, N, D, H, P} tensor configurations")
     ap.add_argument("--output", type=str, default=None, help="result file (default ./<variant>_<model>.json)")
+    ap.add_argument("--ir", type=str, default=None,
+                    help="Path to the IR expressions file (`id: expression` lines): each candidate is recognised and timed")
+    ap.add_argument("--start", type=int, default=0, help="Start from test case ID")
+    ap.add_argument("--num", type=int, default=10, help="Number of expressions to benchmark")
+    ap.add_argument("--end", action="store_true", help="Run from start ID to the last test case")
+    ap.add_argument("--topk", type=int, default=5, help="Number of top kernels to report")
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--runs", type=int, default=100)
     a = ap.parse_args(argv)
@@ -137,10 +181,13 @@ def main(argv=None) -> int:
             ap.error("--configs: expected a JSON list of objects with M, N, D, P (and optionally H)")
     else:
         cfgs = [dict(shapes.DECODE_LLAMA if a.model == "llama" else shapes.DECODE_FALCON)]
+    cands = candidates_from_ir(a.ir, a.start, None if a.end else a.num) if a.ir else None
     out = a.output or f"./{a.variant}_{a.model}.json"
     with open(out, "w") as f:               # the reference starts a run from an empty list (:476)
         json.dump([], f)
-    run(a.variant, cfgs, out, a.warmup, a.runs)
+    records = run(a.variant, cfgs, out, a.warmup, a.runs, cands)
+    if cands is not None:
+        print_report(records, a.topk)
     return 0
 
 

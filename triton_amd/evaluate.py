@@ -155,6 +155,8 @@ def main(argv=None) -> int:
     ap.add_argument("--t", type=str, default="vanilla", help="RMS Type")
     ap.add_argument("--o", type=int, default=0, help="0 only resolve the module, 1 only test, 2 both")
     ap.add_argument("--json", type=str, default=None, help="also write the test result to this file")
+    ap.add_argument("--case", type=str, default=None,
+                    help="IR case file (the reference reads ./evaluation/<t>/<t>_<m>_case<n>.txt): checked to be a candidate of --t")
     a = ap.parse_args(argv)
     if a.t not in VARIANTS:
         ap.error(f"--t: expected one of {VARIANTS}")
@@ -164,6 +166,14 @@ def main(argv=None) -> int:
         ap.error("--o: expected 0, 1 or 2")
     cfg = constants(a.m)
     print(f"[Case{a.n}]")
+    if a.case:
+        from . import ir
+        with open(a.case) as f:
+            m = ir.recognise(f.read().strip())
+        if m.variant != a.t:
+            print(f"Error: {a.case} is not a {a.t} candidate: " + (f"recognised as {m.variant}" if m else m.reason))
+            return 2
+        print(f"{a.case}: {m.variant} ({m.reason})")
     if a.o in (0, 2):
         convert(a.t, cfg)
     if a.o in (1, 2):
