@@ -1,10 +1,15 @@
-// Fused RMSNorm + Q/K/V projection GEMM, 256-token x 256-column workgroup tiles (large problems).
+// Fused RMSNorm + Q/K/V projection GEMM, 256-token x 256- or 192-column workgroup tiles (large problems).
 //
 // Same arithmetic and MFMA mapping as the 128 x 128 kernel (C^T = W^T X^T with 32x32x16 fp16 MFMAs, a lane owns
 // one token), re-balanced for what limits a large GEMM on this chip:
 //   * 4 waves, one per SIMD, each a 128-token x 128-column sub-tile (4 x 4 MFMA blocks, 256 accumulator
 //     registers -- the whole AGPR file of a wave that has its SIMD to itself): every 16-byte LDS operand feeds
-//     four MFMAs instead of two, so LDS bytes and LDS instructions per MFMA are halved.
+//     four MFMAs instead of two, so LDS bytes and LDS instructions per MFMA are halved.  With NB = 3 the sub-tile
+//     is 128 x 96 and the workgroup tile 256 x 192: three quarters of the work per tile, for problems whose
+//     256-wide tiles would fill only three quarters of the chip (2048 tokens x 6144 columns: 192 tiles on 256 CUs).
+//   * The columns of Q, K and V form one axis of 64-column groups (each output padded to whole groups); a tile is
+//     NB consecutive groups and may straddle two outputs: every group has its own buffer descriptor, and every
+//     32-column block of the epilogue its own output.
 //   * Both operands go straight from global memory into LDS (buffer_load ... lds, XOR-swizzled rows); no
 //     register staging and no LDS writes from the VALU.  gamma is multiplied into the X operand after it is read
 //     back from LDS (one packed fp16 multiply per pair: the correctly rounded product), and the waves of the
@@ -18,8 +23,14 @@
 
 namespace trn {
 
-[[maybe_unused]] constexpr int WM = 256, WN = 256, WK = 32;
+[[maybe_unused]] constexpr int WM = 256, WK = 32, WG = 64;       // tokens per tile, contraction columns per stage, columns per group
 
+// Chunk swizzle of a W group row (eight 16-byte chunks, 128 bytes: consecutive rows alternate between the two
+// halves of the 64 banks): with bit 2 from row bit 1 and the low bits from row bits 2-3, the four consecutive rows
+// x four consecutive chunks of one phase of the transposing read touch every bank once.
+__device__ __forceinline__ int gswz(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
+
+template <int NB>
 __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
     // One array per stage and operand: the compiler orders LDS reads after outstanding global->LDS loads that may
@@ -28,6 +39,7 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     __shared__ __attribute__((aligned(1024))) half_t Xs1[WM * WK];
     __shared__ __attribute__((aligned(1024))) half_t Xs2[WM * WK];
     __shared__ __attribute__((aligned(1024))) half_t Xs3[WM * WK];
+    constexpr int WN = NB * WG;                        // columns per tile; a W stage is NB groups of [32 rows][64 columns]
     __shared__ __attribute__((aligned(1024))) half_t Ws0[WK * WN];
     __shared__ __attribute__((aligned(1024))) half_t Ws1[WK * WN];
     __shared__ __attribute__((aligned(1024))) half_t Ws2[WK * WN];
@@ -43,24 +55,28 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
     const int mt = local % a.n_mtiles, nt_all = xcd * a.panels_per_xcd + local / a.n_mtiles;
     if (nt_all >= a.n_panels) return;
-    const int pi = nt_all >= a.p[2].tile0 ? 2 : (nt_all >= a.p[1].tile0 ? 1 : 0);
-    const ProjOut P = a.p[pi];
-    const int n0 = (nt_all - P.tile0) * WN, m0 = mt * WM;
+    const int g_first = nt_all * NB, m0 = mt * WM;      // first column group of the tile
     const int nk = (a.K + WK - 1) / WK;
     constexpr int kOut = 0x7ffffff0;                  // a byte offset past every buffer: the load returns zeros
 
-    // ---- W stage: 32 rows x 512 bytes.  A wave-wide load covers 2 rows; load i of this wave covers stage rows
-    // 16*(i/2) + 8*(i%2) + 2*wave + lane/32: the swizzle depends on row % 16, so two per-lane offsets serve the four.
-    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)P.w, 0, (int)(((int64_t)(a.K - 1) * P.ldw + P.n) * 2), 0x00020000);
-    int w_vo[2];
+    // ---- W stage: per group 32 rows x 128 bytes.  A wave-wide load covers 8 rows of one group; this wave loads rows
+    // 8*wave + lane/8 of every group.  A group belongs to one output: its own descriptor, column offset and pitch.
+    // (Columns of a ragged last group past the output's width read the next row or zeros; they are never stored.)
+    __amdgpu_buffer_rsrc_t wrs[NB];
+    int w_vo[NB], w_tile[NB];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int r = 8 * i + 2 * wave + (lane >> 5);
-        const int chunk = (lane & 16) | ((lane & 15) ^ wswz(r));
-        w_vo[i] = (int)(r * P.ldw * 2) + (n0 + 8 * chunk) * 2;
+    for (int g = 0; g < NB; ++g) {
+        const int gg = g_first + g;
+        const int pi = gg >= a.p[2].tile0 ? 2 : (gg >= a.p[1].tile0 ? 1 : 0);
+        const half_t* w = pi == 2 ? a.p[2].w : pi == 1 ? a.p[1].w : a.p[0].w;
+        const int64_t ldw = pi == 2 ? a.p[2].ldw : pi == 1 ? a.p[1].ldw : a.p[0].ldw;
+        const int n = pi == 2 ? a.p[2].n : pi == 1 ? a.p[1].n : a.p[0].n;
+        const int t0 = pi == 2 ? a.p[2].tile0 : pi == 1 ? a.p[1].tile0 : 0;
+        wrs[g] = __builtin_amdgcn_make_buffer_rsrc((void*)w, 0, (int)(((int64_t)(a.K - 1) * ldw + n) * 2), 0x00020000);
+        const int r = 8 * wave + (lane >> 3);
+        w_vo[g] = (int)(r * ldw * 2) + ((gg - t0) * WG + 8 * ((lane & 7) ^ gswz(r))) * 2;
+        w_tile[g] = (int)(WK * ldw * 2);
     }
-    const int w_row16 = (int)(16 * P.ldw * 2), w_tile = (int)(WK * P.ldw * 2);
     // ---- X stage: 256 rows x 64 bytes, chunk c of row r stored at position c ^ ((r/4) % 4).  A wave-wide load
     // covers 16 rows; load i of this wave covers rows 64*i + 16*wave + lane/4.
     const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
@@ -72,17 +88,18 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
         const int t = m0 + 64 * i + 16 * wave + (lane >> 2);
         x_vo[i] = t < a.T ? (int)(t * a.ldx * 2) + x_chunk * 16 : kOut;          // rows past the end read as zeros
     }
-    // load pair i_ (one X, one W wave-wide load) of stage kt_; columns past hidden hold the next row's data in
-    // X: read zeros instead; W rows past hidden are out of range by themselves
+    // load pair i_ (one X wave-wide load and, for i_ < NB, the W load of group i_) of stage kt_; columns past
+    // hidden hold the next row's data in X: read zeros instead; W rows past hidden are out of range by themselves
 #define TRN_FETCH_ONE(kt_, xd_, wd_, i_)                                                                         \
     do {                                                                                                         \
         const bool drop_ = (kt_) * WK + 8 * x_chunk >= a.K;                                                      \
         __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                                \
             xrs, (__attribute__((address_space(3))) void*)(&xd_[(64 * (i_) + 16 * wave) * WK]), 16,              \
             drop_ ? kOut : x_vo[i_], (kt_) * WK * 2, 0, 0);                                                      \
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                                \
-            wrs, (__attribute__((address_space(3))) void*)(&wd_[(16 * ((i_) >> 1) + 8 * ((i_) & 1) + 2 * wave) * WN]), \
-            16, w_vo[(i_) & 1], (kt_) * w_tile + ((i_) >> 1) * w_row16, 0, 0);                                   \
+        if ((i_) < NB)                                                                                           \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                            \
+                wrs[(i_) < NB ? (i_) : 0], (__attribute__((address_space(3))) void*)(&wd_[((i_) * WK + 8 * wave) * WG]), 16, \
+                w_vo[(i_) < NB ? (i_) : 0], (kt_) * w_tile[(i_) < NB ? (i_) : 0], 0, 0);                         \
     } while (0)
 #define TRN_FETCH(kt_, xd_, wd_) _Pragma("unroll") for (int fi_ = 0; fi_ < 4; ++fi_) TRN_FETCH_ONE(kt_, xd_, wd_, fi_)
 
@@ -107,43 +124,43 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) xoff[ks] = (wm * 128 + c) * WK + (((2 * ks + h) ^ ((c >> 2) & 3)) << 3);
     // W^T A-operand via the transposing read: lane's piece is stage row ks*16 + 8h + (lane%16)/4 [+4], columns
-    // wn*128 + nb*32 + 16*((lane/16)%2) + 4*(lane%4)
-    int woff_lo[4], woff_hi[4];
+    // (wn*NB + nb)*32 + 16*((lane/16)%2) + 4*(lane%4) of the tile, i.e. group (wn*NB + nb)/2, chunks 4*((wn*NB + nb)%2) ..
+    int woff_lo[NB], woff_hi[NB];
     {
         const int rl = 8 * h + ((lane & 15) >> 2), rh = rl + 4;
         const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), sub = (lane & 1) * 4;
 #pragma unroll
-        for (int nb = 0; nb < 4; ++nb) {
-            const int chunk = wn * 16 + nb * 4 + lc;
-            woff_lo[nb] = rl * WN + ((chunk ^ wswz(rl)) << 3) + sub;
-            woff_hi[nb] = rh * WN + ((chunk ^ wswz(rh)) << 3) + sub;
+        for (int nb = 0; nb < NB; ++nb) {
+            const int blk = wn * NB + nb, chunk = 4 * (blk & 1) + lc;
+            woff_lo[nb] = (blk >> 1) * WK * WG + rl * WG + ((chunk ^ gswz(rl)) << 3) + sub;
+            woff_hi[nb] = (blk >> 1) * WK * WG + rh * WG + ((chunk ^ gswz(rh)) << 3) + sub;
         }
     }
-    half8_t xb0[4], xb1[4], wa0[4], wa1[4];           // operands of the two contraction steps of a k-tile
+    half8_t xb0[4], xb1[4], wa0[NB], wa1[NB];           // operands of the two contraction steps of a k-tile
     auto read_x = [&](const half_t* Xc, int ks, int mb) __attribute__((always_inline)) {
         return *reinterpret_cast<const half8_t*>(&Xc[xoff[ks] + mb * 32 * WK]);
     };
     auto read_w = [&](const half_t* Wc, int ks, int nb) __attribute__((always_inline)) {
-        const half4_t lo = lds_read_tr16(&Wc[ks * 16 * WN + woff_lo[nb]]);
-        const half4_t hi = lds_read_tr16(&Wc[ks * 16 * WN + woff_hi[nb]]);
+        const half4_t lo = lds_read_tr16(&Wc[ks * 16 * WG + woff_lo[nb]]);
+        const half4_t hi = lds_read_tr16(&Wc[ks * 16 * WG + woff_hi[nb]]);
         return half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
     };
 
-    float16_t acc[4][4];   // [column block][token block]
+    float16_t acc[NB][4];   // [column block][token block]
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.f;
     float ss[4] = {0.f, 0.f, 0.f, 0.f};
-    // One contraction step = 4 groups (one token block each) of 4 MFMAs.  A wave has its SIMD to itself, so
+    // One contraction step = 4 groups (one token block each) of NB MFMAs.  A wave has its SIMD to itself, so
     // whatever else it issues must sit between MFMAs or the pipe runs dry: every MFMA heads a slot that also
     // carries a piece of the other work -- the sum of squares and gamma multiply of the NEXT group's operand
     // (the next step's first one in the last group), the next step's operand reads (W operands first: its first
-    // group needs all four), and, in the second step of a k-tile, a quarter of the stage refill.
-    auto step = [&](half8_t& xv, half8_t (&xb)[4], half8_t (&wa)[4], const half8_t& g, half8_t (&xn)[4],
-                    half8_t (&wn_)[4], const half_t* Xr, const half_t* Wr, int ks_r, const half8_t& gn,
+    // group needs all of them), and, in the second step of a k-tile, a quarter of the stage refill.
+    auto step = [&](half8_t& xv, half8_t (&xb)[4], half8_t (&wa)[NB], const half8_t& g, half8_t (&xn)[4],
+                    half8_t (&wn_)[NB], const half_t* Xr, const half_t* Wr, int ks_r, const half8_t& gn,
                     auto&& extra) __attribute__((always_inline)) {
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
@@ -161,13 +178,18 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
                     ss[(mb + 1) & 3] = __builtin_amdgcn_fdot2(p, p, ss[(mb + 1) & 3], false);
                 }
             }
+            if constexpr (NB == 3) {
+                if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
+            }
             __builtin_amdgcn_sched_barrier(0);
             acc[2][mb] = mfma32(wa[2], xv, acc[2][mb]);
             const half8_t xv_next = raw * (mb < 3 ? g : gn);
-            if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
-            if (mb == 1) wn_[3] = read_w(Wr, ks_r, 3);
-            __builtin_amdgcn_sched_barrier(0);
-            acc[3][mb] = mfma32(wa[3], xv, acc[3][mb]);
+            if constexpr (NB == 4) {
+                if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
+                if (mb == 1) wn_[3] = read_w(Wr, ks_r, 3);
+                __builtin_amdgcn_sched_barrier(0);
+                acc[3][mb] = mfma32(wa[3], xv, acc[3][mb]);
+            }
             if (mb < 2) xn[mb] = read_x(Xr, ks_r, mb);
             extra(mb);
             __builtin_amdgcn_sched_barrier(0);
@@ -187,7 +209,9 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0)
     __syncthreads();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { xb0[i] = read_x(Xs0, 0, i); wa0[i] = read_w(Ws0, 0, i); }
+    for (int i = 0; i < 4; ++i) xb0[i] = read_x(Xs0, 0, i);
+#pragma unroll
+    for (int i = 0; i < NB; ++i) wa0[i] = read_w(Ws0, 0, i);
     half8_t xv = xb0[0];                    // the operand of the next MFMA group, gamma applied
     if (stats) {
 #pragma unroll
@@ -205,9 +229,11 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
                      const half8_t (&gn)[2], half8_t (&gf)[2]) __attribute__((always_inline)) {
         step(xv, xb0, wa0, gc[0], xb1, wa1, Xc, Wc, 1, gc[1], [&](int) __attribute__((always_inline)) {});
         // Stage kt+1 must have landed.  Loads complete in issue order, and behind this wave's share of that stage
-        // only the refills and gamma slices of the last two k-tiles (2 x (8 + 2) loads) have been issued.
+        // only the refills and gamma slices of the last two k-tiles (2 x (4 + NB + 2) loads) have been issued.
         // lgkmcnt(0): this wave's reads of stage kt have returned, so the refill cannot overtake them.
-        if (use_g) __builtin_amdgcn_s_waitcnt(0x4074); else __builtin_amdgcn_s_waitcnt(0x4070);
+        constexpr int kBehindG = 2 * (4 + NB + 2), kBehind = 2 * (4 + NB);
+        if (use_g) __builtin_amdgcn_s_waitcnt(0x0070 | (kBehindG & 15) | ((kBehindG >> 4) << 14));
+        else __builtin_amdgcn_s_waitcnt(0x0070 | (kBehind & 15) | ((kBehind >> 4) << 14));
         // A bare barrier: __syncthreads() would first drain every load in flight, the prefetched stages included.
         // Nothing else needs ordering here -- in this loop LDS is written only by those loads.
         __builtin_amdgcn_s_barrier();       // everyone's share landed; nobody still reads stage kt
@@ -237,42 +263,44 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     }
     __syncthreads();                        // also: every wave is done with the stages
 
-    // ---- epilogue: scale, transpose 64 tokens x 64 columns at a time through LDS (two stage arrays of 16 KB
-    // per wave, used alternately), store 16 bytes per lane: 8 lanes cover the 64 columns of a token, 8 tokens per
-    // store instruction
+    // ---- epilogue: scale, transpose 64 tokens x 32 columns at a time through LDS (this wave's own X stage),
+    // store 16 bytes per lane: 4 lanes cover the 32 columns of a token, 16 tokens per store instruction.  A
+    // 32-column block lies in one group, hence in one output and (head_dim being a multiple of 32) in one head.
     {
-        constexpr int OP = 64 + 4;                          // pitch in halfs; 64*68*2 = 8704 bytes <= a stage
+        constexpr int OP = 32 + 8;                          // pitch in halfs
         half_t* ot = wave == 0 ? Xs0 : wave == 1 ? Xs1 : wave == 2 ? Xs2 : Xs3;
-        const int orow = lane >> 3, ocol = (lane & 7) * 8;
+        const int orow = lane >> 2, ocol = (lane & 3) * 8;
 #pragma unroll
-        for (int p = 0; p < 2; ++p) {
-            float r[2];
+        for (int nb = 0; nb < NB; ++nb) {
+            const int blk = wn * NB + nb, gg = g_first + (blk >> 1);
+            const int pi = gg >= a.p[2].tile0 ? 2 : (gg >= a.p[1].tile0 ? 1 : 0);
+            half_t* out = pi == 2 ? a.p[2].out : pi == 1 ? a.p[1].out : a.p[0].out;
+            const int64_t stride_h = pi == 2 ? a.p[2].stride_h : pi == 1 ? a.p[1].stride_h : a.p[0].stride_h;
+            const int64_t stride_s = pi == 2 ? a.p[2].stride_s : pi == 1 ? a.p[1].stride_s : a.p[0].stride_s;
+            const int pn = pi == 2 ? a.p[2].n : pi == 1 ? a.p[1].n : a.p[0].n;
+            const int t0 = pi == 2 ? a.p[2].tile0 : pi == 1 ? a.p[1].tile0 : 0;
+            const int n = (gg - t0) * WG + (blk & 1) * 32 + ocol;
+            half_t* obase = out + (int64_t)(n / a.head_dim) * stride_h + (n % a.head_dim);
 #pragma unroll
-            for (int ml = 0; ml < 2; ++ml) r[ml] = a.norm ? rstd_s[wm * 128 + (2 * p + ml) * 32 + c] : 1.0f;
+            for (int p = 0; p < 2; ++p) {
 #pragma unroll
-            for (int q = 0; q < 2; ++q) {
+                for (int ml = 0; ml < 2; ++ml) {
+                    const float r = a.norm ? rstd_s[wm * 128 + (2 * p + ml) * 32 + c] : 1.0f;
 #pragma unroll
-                for (int ml = 0; ml < 2; ++ml)
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        half4_t ov;
 #pragma unroll
-                    for (int nl = 0; nl < 2; ++nl)
-#pragma unroll
-                        for (int r4 = 0; r4 < 4; ++r4) {
-                            half4_t ov;
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) ov[e] = (half_t)(acc[2 * q + nl][2 * p + ml][r4 * 4 + e] * r[ml]);
-                            *reinterpret_cast<half4_t*>(&ot[(ml * 32 + c) * OP + nl * 32 + 8 * r4 + 4 * h]) = ov;
-                        }
+                        for (int e = 0; e < 4; ++e) ov[e] = (half_t)(acc[nb][2 * p + ml][r4 * 4 + e] * r);
+                        *reinterpret_cast<half4_t*>(&ot[(ml * 32 + c) * OP + 8 * r4 + 4 * h]) = ov;
+                    }
+                }
                 // (LDS operations of one wave execute in order: its reads below see its writes above, and the
                 // next pass's writes come after these reads)
-                const int n = n0 + wn * 128 + q * 64 + ocol;
-                half_t* obase = P.out + (int64_t)(n / a.head_dim) * P.stride_h + (n % a.head_dim);
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int tl = j * 8 + orow, t = m0 + wm * 128 + p * 64 + tl;
-                    const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol]);
-                    const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol + 4]);
-                    if (t < a.T && n < P.n)
-                        *reinterpret_cast<uint4_t*>(obase + (int64_t)t * P.stride_s) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+                for (int j = 0; j < 4; ++j) {
+                    const int tl = j * 16 + orow, t = m0 + wm * 128 + p * 64 + tl;
+                    const uint4_t ov = *reinterpret_cast<const uint4_t*>(&ot[tl * OP + ocol]);
+                    if (t < a.T && n < pn) *reinterpret_cast<uint4_t*>(obase + (int64_t)t * stride_s) = ov;
                 }
             }
         }
@@ -280,21 +308,34 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
 #endif
 }
 
+// Tiles of nb 64-column groups over the group axis [Q | K | V], each output padded to whole groups.
+static int64_t wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv, int nb) {
+    const int64_t groups = (n_q + WG - 1) / WG + 2 * ((n_kv + WG - 1) / WG);
+    return ((tokens + WM - 1) / WM) * ((groups + nb - 1) / nb);
+}
+
+// 192-column tiles when they keep the chip busier: the time is (rounds of 256 workgroups) x (work per tile), and a
+// 192-wide tile does 3/4 of the work of a 256-wide one at slightly lower efficiency (fewer MFMAs per operand read).
+static bool narrow_is_better(int64_t tokens, int64_t n_q, int64_t n_kv) {
+    const int64_t r4 = (wide_tiles(tokens, n_q, n_kv, 4) + 255) / 256, r3 = (wide_tiles(tokens, n_q, n_kv, 3) + 255) / 256;
+    return r3 * 3 * 100 < r4 * 4 * 95;
+}
+
 int launch_prenorm_qkv_wide(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream) {
+    const int nb = narrow_is_better(a.T, n_q, n_kv) ? 3 : 4;
     a.n_mtiles = (a.T + WM - 1) / WM;
-    const int tq = (int)((n_q + WN - 1) / WN), tkv = (int)((n_kv + WN - 1) / WN);
-    a.p[0].tile0 = 0; a.p[1].tile0 = tq; a.p[2].tile0 = tq + tkv;
-    a.n_panels = tq + 2 * tkv;
+    const int gq = (int)((n_q + WG - 1) / WG), gkv = (int)((n_kv + WG - 1) / WG);
+    a.p[0].tile0 = 0; a.p[1].tile0 = gq; a.p[2].tile0 = gq + gkv;      // first group of each output
+    a.n_panels = (gq + 2 * gkv + nb - 1) / nb;
     a.panels_per_xcd = (a.n_panels + 7) / 8;
     const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
     if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
-    hipLaunchKernelGGL(prenorm_qkv_wide_kernel, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    if (nb == 3) hipLaunchKernelGGL(prenorm_qkv_wide_kernel<3>, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(prenorm_qkv_wide_kernel<4>, dim3((unsigned)grid), dim3(256), 0, stream, a);
     return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }
 
-// Workgroups the wide tiling would launch (useful ones, not counting the padding of the XCD mapping).
-int64_t prenorm_qkv_wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv) {
-    return ((tokens + WM - 1) / WM) * ((n_q + WN - 1) / WN + 2 * ((n_kv + WN - 1) / WN));
-}
+// Workgroups the 256-column tiling would launch (useful ones, not counting the padding of the XCD mapping).
+int64_t prenorm_qkv_wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv) { return wide_tiles(tokens, n_q, n_kv, 4); }
 
 }  // namespace trn
