@@ -15,8 +15,8 @@
 // Q tiles of 64 queries go straight from global memory into a ring of three LDS stages (buffer_load ... lds,
 // XOR-swizzled rows), requested two tiles ahead, one barrier per tile.  What the VALU needs per tile besides the scores -- the row
 // normalisers and, for KeyFormer, the wave's 64 x 32 block of fp32 noise, which is the HBM stream that bounds
-// that variant -- is loaded into registers one whole tile ahead, so that a CU always has about 64 KB of noise
-// in flight.  All of these loads are buffer loads with out-of-range zero fill and are issued unconditionally
+// that variant -- is loaded into registers one to two tiles ahead (a block's registers are refilled as soon as it
+// has been consumed), so that a CU has 64 - 128 KB of noise in flight.  All of these loads are buffer loads with out-of-range zero fill and are issued unconditionally
 // in a fixed order: the wait for a Q stage counts the loads issued behind it.  Masks (causal diagonal, ragged
 // ends) are evaluated only in the blocks that need them (a wave-uniform test).
 #include "common.h"
@@ -38,7 +38,9 @@ struct ColArgs {
 constexpr int CBN = 128;  // keys per workgroup
 [[maybe_unused]] constexpr int CBM = 64;   // queries per staged tile
 
-template <int D, bool NOISE>
+// SQ: the sums of squares are wanted too (RoCo); without them (KeyFormer) their accumulators and one of the five
+// VALU operations per score are not compiled in.
+template <int D, bool NOISE, bool SQ>
 __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const ColArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
     constexpr int NKS = D / 16;
@@ -48,6 +50,9 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
     __shared__ __attribute__((aligned(1024))) half_t Qs0[CBM * D];
     __shared__ __attribute__((aligned(1024))) half_t Qs1[CBM * D];
     __shared__ __attribute__((aligned(1024))) half_t Qs2[CBM * D];
+    // KeyFormer: the wave's 32 x 32 block of noise is fetched with whole 128-byte row pieces per 8 lanes (a load
+    // instruction then touches 8 cache lines, not 32) and turned into the accumulator layout through this array
+    __shared__ __attribute__((aligned(1024))) float Ns[NOISE ? 4 * 1024 : 4];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -70,9 +75,9 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
         for (int ks = 0; ks < NKS; ++ks) kA[ks] = *reinterpret_cast<const half8_t*>(kp + ks * 16);
     }
 
-    float s1[16], s2[16];
+    float s1[16], s2[SQ ? 16 : 1];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { s1[r] = 0.f; s2[r] = 0.f; }
+    for (int r = 0; r < 16; ++r) { s1[r] = 0.f; if constexpr (SQ) s2[r] = 0.f; }
 
     // ---- Q stages: direct global -> LDS; queries past the end read as zeros
     const __amdgpu_buffer_rsrc_t qrs = __builtin_amdgcn_make_buffer_rsrc(
@@ -92,20 +97,31 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
     const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(NOISE ? a.noise + b * a.nb + head * a.nh : a.lse), 0,
         NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
-    const int nvo = NOISE ? (int)((c * a.ns + wkey0 + 4 * h) * 4) : 0;   // lane's query row, first 4 keys of its 16
-    struct Pre { float lse[2]; float4_t g[2][4]; };
-    Pre pc, pn;      // this tile's values and the next one's
-    auto prefetch = [&](int t, Pre& p) __attribute__((always_inline)) {
+    // load i of a block covers its query rows 8i .. 8i+7: lane -> row 8i + lane/8, keys 4*(lane%8) .. +3
+    const int nvo = NOISE ? (int)(((lane >> 3) * a.ns + wkey0 + 4 * (lane & 7)) * 4) : 0;
+    const int nrow8 = NOISE ? (int)(8 * a.ns * 4) : 0;
+    // transposer: the 16-byte chunk q of row r sits at chunk r*8 + (q ^ ((r/2) % 8)); written as loaded, read as
+    // row c, chunks 2*r4 + h (both conflict-free)
+    float* nsw = Ns + (NOISE ? wave * 1024 : 0);
+    int ns_wr[4], ns_rd[4];
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb)
-            p.lse[qb] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(lrs, c * 4, (t * CBM + qb * 32) * 4, 0));
+    for (int i = 0; i < 4; ++i) {
+        const int r = 8 * i + (lane >> 3);
+        ns_wr[i] = (r * 8 + ((lane & 7) ^ ((r >> 1) & 7))) * 4;
+        ns_rd[i] = (c * 8 + ((2 * i + h) ^ ((c >> 1) & 7))) * 4;
+    }
+    // Two register buffers, used by even and odd tiles in turn.  A block's half of a buffer is refilled, for the tile
+    // after next, as soon as that block has been consumed, so between one and two tiles of noise (8 - 16 KB per
+    // wave) are in flight at any time.
+    struct Pre { float lse[2]; float4_t g[2][4]; };
+    Pre pa, pb;
+    auto prefetch = [&](int t, int qb, Pre& p) __attribute__((always_inline)) {
+        p.lse[qb] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(lrs, c * 4, (t * CBM + qb * 32) * 4, 0));
         if constexpr (NOISE) {
 #pragma unroll
-            for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4)
-                    p.g[qb][r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
-                        nrs, nvo + r4 * 32, (int)((t * CBM + qb * 32) * a.ns * 4), 0));
+            for (int r4 = 0; r4 < 4; ++r4)
+                p.g[qb][r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(
+                    nrs, nvo + r4 * nrow8, (int)((t * CBM + qb * 32) * a.ns * 4), 0));
         }
     };
 
@@ -114,8 +130,15 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
 
     // The VALU part of a 32-query block.  Masked and plain blocks are separate loops (one wave-uniform branch
     // per block) so that the plain one is 4 instructions per score: fma, exp2, add, fma.
-    auto softmax_sums = [&](const float16_t& acc, int qfirst, float lse, const float4_t (&gq)[4]) __attribute__((always_inline)) {
+    auto softmax_sums = [&](const float16_t& acc, int qfirst, float lse, const float4_t (&gl)[4]) __attribute__((always_inline)) {
         const float lse2 = lse * kLog2e;
+        float4_t gq[4];
+        if constexpr (NOISE) {       // (LDS operations of one wave execute in order: no barrier between the two)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *reinterpret_cast<float4_t*>(&nsw[ns_wr[i]]) = gl[i];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) gq[i] = *reinterpret_cast<const float4_t*>(&nsw[ns_rd[i]]);
+        }
         const bool masked = (qfirst + 31 >= a.Sq) || (wkey0 + 31 >= a.Skv) || (a.causal && wkey0 + 31 > qfirst + off);
         if (masked) {
             // last key this lane's query may count, as an offset from the lane's first key (-1: none)
@@ -127,7 +150,7 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
                 if constexpr (NOISE) t = __builtin_fmaf(gq[r / 4][r % 4], a.c3, t);
                 const float p = (8 * (r / 4) + (r % 4) <= last) ? fast_exp2(t) : 0.f;
                 s1[r] += p;
-                s2[r] = __builtin_fmaf(p, p, s2[r]);
+                if constexpr (SQ) s2[r] = __builtin_fmaf(p, p, s2[r]);
             }
         } else {
 #pragma unroll
@@ -136,67 +159,74 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
                 if constexpr (NOISE) t = __builtin_fmaf(gq[r / 4][r % 4], a.c3, t);
                 const float p = fast_exp2(t);
                 s1[r] += p;
-                s2[r] = __builtin_fmaf(p, p, s2[r]);
+                if constexpr (SQ) s2[r] = __builtin_fmaf(p, p, s2[r]);
             }
         }
     };
     // The two 32-query blocks of a tile.  Each block's eight score MFMAs accumulate into one register block (a
     // dependent chain); all operands of a chain are in registers before it starts, and the second block's are
     // read while the first chain runs.
-    auto blocks = [&](const half_t* Qc, int q0, const Pre& pc) __attribute__((always_inline)) {
+    auto blocks = [&](const half_t* Qc, int t, Pre& pc) __attribute__((always_inline)) {
+        const int q0 = t * CBM;
         // (causal) none of a block's queries sees any of this wave's keys: skip it
         const bool live0 = !(a.causal && q0 + 31 + off < wkey0), live1 = !(a.causal && q0 + 63 + off < wkey0);
-        if (!live1) return;
         float16_t acc0, acc1;
+        if (live1) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
-        half8_t qa[NKS];
+            for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+            half8_t qa[NKS];
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[qoff[ks]]);
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-            acc0 = mfma32(kA[ks], qa[ks], acc0);
-            qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[32 * D + qoff[ks]]);
+            for (int ks = 0; ks < NKS; ++ks) qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[qoff[ks]]);
             __builtin_amdgcn_sched_barrier(0);
-        }
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) acc1 = mfma32(kA[ks], qa[ks], acc1);
-        __builtin_amdgcn_sched_barrier(0);
-        if (live0) softmax_sums(acc0, q0, pc.lse[0], pc.g[0]);
-        softmax_sums(acc1, q0 + 32, pc.lse[1], pc.g[1]);
+            for (int ks = 0; ks < NKS; ++ks) {
+                acc0 = mfma32(kA[ks], qa[ks], acc0);
+                qa[ks] = *reinterpret_cast<const half8_t*>(&Qc[32 * D + qoff[ks]]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) acc1 = mfma32(kA[ks], qa[ks], acc1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (live0) softmax_sums(acc0, q0, pc.lse[0], pc.g[0]);
+        }
+        prefetch(t + 2, 0, pc);              // (unconditional, like every load of the loop: see below)
+        if (live1) softmax_sums(acc1, q0 + 32, pc.lse[1], pc.g[1]);
+        prefetch(t + 2, 1, pc);
     };
-    // tile t: its stage has landed once this wave's own share has (everything issued behind it is the
-    // prefetch of the same tile: 2 normaliser loads and, with noise, 8 noise loads) and the others' too
     // Tile t reads stage t % 3; the stage of tile t+2 is requested as soon as the barrier shows that everybody has
-    // left tile t-1 (its previous tenant), so a Q stage has two tile times to arrive from L2.  Behind this wave's
-    // share of stage t only the register prefetch of tile t and stage t+1 have been issued: NI + 2 (+ 8 with noise)
-    // requests.  All of them are issued unconditionally (past the last tile everything reads as zeros into a stage
-    // nobody uses): the compiler sizes its own waits for prefetched registers by the loads it KNOWS follow them, and
-    // a conditional load counts as absent, which would make every use of a prefetched value drain the refills too.
-    auto tile = [&](int t, const half_t* Qc, half_t* Qf) __attribute__((always_inline)) {
-        constexpr int kBehind = NI + 2 + (NOISE ? 8 : 0);
+    // left tile t-1 (its previous tenant), so a Q stage has two tile times to arrive from L2.  Tile t's stage has
+    // landed once this wave's own share has, and the others' too.  Behind this wave's share of stage t these have
+    // been issued, in this order: the register prefetch of tile t (during tile t-2), stage t+1, the register
+    // prefetch of tile t+1 (during tile t-1): NI + 4 requests (+ 16 with noise).  All of them are issued
+    // unconditionally (past the last tile everything reads as zeros, the stages into one nobody uses): the compiler
+    // sizes its own waits for prefetched registers by the loads it KNOWS follow them, and a conditional load counts
+    // as absent, which would make every use of a prefetched value drain the refills too.
+    auto tile = [&](int t, const half_t* Qc, half_t* Qf, Pre& pc) __attribute__((always_inline)) {
+        constexpr int kBehind = NI + 4 + (NOISE ? 16 : 0);
         __builtin_amdgcn_s_waitcnt(0x0f70 | (kBehind & 15) | ((kBehind >> 4) << 14));
         __builtin_amdgcn_s_barrier();        // (a bare barrier: nothing else in flight needs draining)
         __builtin_amdgcn_sched_barrier(0);
-        prefetch(t + 1, pn);
         TRN_FETCH_Q(t + 2, Qf);
         __builtin_amdgcn_sched_barrier(0);
-        blocks(Qc, t * CBM, pc);
-        pc = pn;                             // (waits for the register prefetch only: the stage request is behind it)
+        blocks(Qc, t, pc);
     };
+    // the same order of requests as in the loop, so that the count above holds from the first tile on
     TRN_FETCH_Q(t0, Qs0);
-    prefetch(t0, pc);
+    prefetch(t0, 0, pa); prefetch(t0, 1, pa);
     TRN_FETCH_Q(t0 + 1, Qs1);
+    prefetch(t0 + 1, 0, pb); prefetch(t0 + 1, 1, pb);
     // Pin the arrival of the K rows here, ahead of the loop.  Left to the first MFMA that reads them, the wait the
     // compiler inserts sits inside the loop body and, being conservative across the back edge, drains the stage and
     // prefetch loads of every iteration.
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) asm volatile("" ::"v"(kA[ks]));
-    for (int t = t0; t < nt; t += 3) {
-        tile(t, Qs0, Qs2);
-        if (t + 1 < nt) tile(t + 1, Qs1, Qs0);
-        if (t + 2 < nt) tile(t + 2, Qs2, Qs1);
+    for (int t = t0; t < nt; t += 6) {       // three stages x two register buffers
+        tile(t, Qs0, Qs2, pa);
+        if (t + 1 < nt) tile(t + 1, Qs1, Qs0, pb);
+        if (t + 2 < nt) tile(t + 2, Qs2, Qs1, pa);
+        if (t + 3 < nt) tile(t + 3, Qs0, Qs2, pb);
+        if (t + 4 < nt) tile(t + 4, Qs1, Qs0, pa);
+        if (t + 5 < nt) tile(t + 5, Qs2, Qs1, pb);
     }
 #undef TRN_FETCH_Q
 
@@ -204,13 +234,13 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
     const int64_t obase = ((int64_t)b * a.Hq + head) * a.Skv;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        float x = s1[r], y = s2[r];
+        float x = s1[r], y = SQ ? s2[SQ ? r : 0] : 0.f;
 #pragma unroll
-        for (int msk = 1; msk < 32; msk <<= 1) { x += __shfl_xor(x, msk, 64); y += __shfl_xor(y, msk, 64); }
+        for (int msk = 1; msk < 32; msk <<= 1) { x += __shfl_xor(x, msk, 64); if constexpr (SQ) y += __shfl_xor(y, msk, 64); }
         const int key = wkey0 + 8 * (r / 4) + 4 * h + (r % 4);
         if (c == 0 && key < a.Skv) {
             if (a.out_sum) a.out_sum[obase + key] = x;
-            if (a.out_sumsq) a.out_sumsq[obase + key] = y;
+            if (SQ && a.out_sumsq) a.out_sumsq[obase + key] = y;
         }
     }
 #endif
@@ -219,7 +249,8 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
 template <int D, bool NOISE>
 static hipError_t launch_col(const ColArgs& a, hipStream_t s) {
     const unsigned grid = (unsigned)a.n_kvtiles * a.B * a.Hq;
-    hipLaunchKernelGGL((attn_colstats_kernel<D, NOISE>), dim3(grid), dim3(256), 0, s, a);
+    if (a.out_sumsq) hipLaunchKernelGGL((attn_colstats_kernel<D, NOISE, true>), dim3(grid), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((attn_colstats_kernel<D, NOISE, false>), dim3(grid), dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
