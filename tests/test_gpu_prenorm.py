@@ -22,9 +22,12 @@ def weights(g, K, nq, nkv, std=0.02):
 @pytest.mark.parametrize("T,K,nq,nkv,D,norm", [(256, 512, 512, 128, 128, True), (130, 520, 192, 64, 64, True),
                                               (16, 4096, 4096, 4096, 128, False), (2048, 4096, 4096, 1024, 128, True),
                                               (1, 64, 64, 64, 64, True), (16, 4544, 4544, 64, 64, True),
-                                              # 256 x 256 tiling (>= 128 of its tiles): ragged tokens and hidden,
-                                              # a nearly empty K/V panel, no norm
+                                              # the wide tilings (>= 128 tiles of 256 x 256): ragged tokens and hidden, a
+                                              # nearly empty K/V group, no norm -- 256 x 192 tiles (the first three: tiles
+                                              # straddle Q | K | V, ragged last tile) and 256 x 256 tiles (the last two)
                                               (1000, 520, 6144, 1024, 128, True), (300, 200, 16384, 64, 64, False),
+                                              (900, 264, 8192 + 64, 192, 64, True),
+                                              (2048, 200, 6144, 1024, 128, True), (1800, 136, 7168 - 64, 512, 64, False),
                                               # at most 32 tokens: the weight-streaming tiling (four waves split hidden)
                                               (32, 520, 1024, 256, 128, True), (5, 72, 192, 64, 64, True),
                                               (17, 8192, 256, 128, 128, True), (33, 520, 256, 128, 128, True)])
@@ -65,7 +68,8 @@ def test_projection_into_kv_cache_rows():
 
 @pytest.mark.parametrize("T,K,nq,nkv,D", [(200, 136, 256, 64, 64),         # 128 x 128 tiling
                                          (20, 136, 320, 64, 64),          # weight-streaming tiling
-                                         (600, 136, 5120, 512, 128)])      # 256 x 256 tiling
+                                         (520, 136, 10240, 512, 128),      # 256 x 192 tiling, tiles straddling Q | K | V
+                                         (2048, 136, 6144, 1024, 128)])    # 256 x 256 tiling
 def test_projection_reads_and_writes_stay_inside_its_views(T, K, nq, nkv, D):
     """Operands are padded views cut out of NaN-filled buffers, hidden and tokens are ragged: a tile load that strays
     past a row or the end of a view pulls NaN into the product, a store that strays overwrites the NaN padding."""
