@@ -111,7 +111,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
     float m = -INFINITY, l = 0.f;      // reference max (log2 domain) and this lane's partial row sum
-    float m2 = -INFINITY, l2 = 0.f;    // same for the perturbed scores
+    float m2 = 0.f, l2 = 0.f;          // same for the perturbed scores: reference (finite; meaningful once have2) and sum
+    bool have2 = false;
 
     int ntiles = (a.Skv + BN - 1) / BN;
     if (a.causal) ntiles = min(ntiles, (min(q0 + BM - 1, a.Sq - 1) + off) / BN + 1);
@@ -160,31 +161,40 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
         // accumulators never meet a control-flow merge.  (Two whole-step variants selected by a branch cost
         // dozens of accumulator register copies per step and broke the in-place MFMA accumulation chains.)
         if constexpr (NOISE) {
-            float zmax = m2;
-            float16_t z;
+            // Row normaliser of the perturbed scores z = s*c2 + g*c3 (log2 domain), with a lazy reference like the
+            // main softmax: d = z - m2 comes straight out of two fused multiply-adds, and m2 is only raised when some d
+            // exceeds 8 (the sum lives in fp32: 2^8 of head-room is harmless) or nothing has been summed yet.
+            const float nref = -m2;
+            float16_t d;
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 const float4_t gv = gpre[r4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float zz = sx[r4 * 4 + e] * a.c2 + gv[e] * a.c3;
+                    float dd = __builtin_fmaf(sx[r4 * 4 + e], a.c2, __builtin_fmaf(gv[e], a.c3, nref));
                     if (masked) {
                         const int key = key0 + 8 * r4 + 4 * h + e;
-                        zz = (key < a.Skv && (!a.causal || key <= qrow + off)) ? zz : -INFINITY;
+                        dd = (key < a.Skv && (!a.causal || key <= qrow + off)) ? dd : -INFINITY;
                     }
-                    z[r4 * 4 + e] = zz;
-                    zmax = fmaxf(zmax, zz);
+                    d[r4 * 4 + e] = dd;
                 }
             }
             fetch_noise(key0 + 64, gpre);    // the next block of the same parity, two pipeline steps ahead of its use
-            zmax = half_max(zmax);
-            if (zmax > -INFINITY) {          // a block can be entirely masked for this row pair
-                float sum = 0.f;
+            const float dmax = half_max(max16(d));             // (shared by the lane pair of a query, like m2)
+            const bool seen = dmax > -INFINITY;                // a block can be entirely masked for this row pair
+            const bool raise = dmax > 8.0f || (!have2 && seen);
+            if (__builtin_amdgcn_ballot_w64(raise) != 0) {     // wave-uniform; rare after a row's first block
+                const float shift = raise ? dmax : 0.f;
+                l2 *= fast_exp2(-shift);
+                m2 += shift;
 #pragma unroll
-                for (int r = 0; r < 16; ++r) sum += fast_exp2(z[r] - zmax);
-                l2 = l2 * fast_exp2(m2 - zmax) + sum;
-                m2 = zmax;
+                for (int r = 0; r < 16; ++r) d[r] -= shift;
             }
+            have2 = have2 || seen;
+            float sum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum += fast_exp2(d[r]);
+            l2 += sum;
         }
         if (masked) {
 #pragma unroll
