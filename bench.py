@@ -228,6 +228,18 @@ def bench_decode(steps, warmup):
             _, ev = graph_timed(m, t, steps, warmup, per_graph=1)
             res[v + "_us"] = round(ev * 1e3, 2)
         out[name] = res
+    # the reference's other two workloads at the first shape its drivers list (lora_benchmark.py:545, gmlp_benchmark.py:53-64)
+    g = torch.Generator(device="cuda").manual_seed(42)
+    rnd = lambda *shape: torch.randn(*shape, device="cuda", generator=g).clamp_(-1, 1).mul_(0.01).half()
+    M, N, P, R = 16, 1024, 512, 64
+    t = dict(X=rnd(M, N), W=rnd(N, P), A=rnd(N, R), B=rnd(R, P), O=torch.zeros(M, P, dtype=torch.float16, device="cuda"))
+    _, ev = graph_timed(modules.get("lora", "linear"), t, steps, warmup, per_graph=1)
+    out["lora_M16_N1024_P512_R64_us"] = round(ev * 1e3, 2)
+    K = 1024
+    t = dict(X=torch.randn(M, K, device="cuda", generator=g).half(), W1=torch.randn(K, N, device="cuda", generator=g).half(),
+             W2=torch.randn(K, N, device="cuda", generator=g).half(), O=torch.zeros(M, N, dtype=torch.float16, device="cuda"))
+    _, ev = graph_timed(modules.get("gmlp", "linear"), t, steps, warmup, per_graph=1)
+    out["gmlp_M16_K1024_N1024_us"] = round(ev * 1e3, 2)
     return out
 
 

@@ -163,6 +163,29 @@ int trn_prenorm_qkv_f16(const void* x, const void* gamma /* nullable */,
                         float eps, int32_t norm, void* stream);
 
 /*
+ * Up to three plain projections of one activation matrix:  out_i = x w_i (+ addend_i),  i < n_mats <= 3, with
+ * x [tokens, hidden], w_i [hidden, n_i], out_i / addend_i [tokens, n_i], all fp16 row-major with the given row
+ * pitches; addend (the array or an entry) may be NULL, and addend_i may be out_i itself.  The product is rounded to
+ * fp16 before the addend is added, as two separate GEMMs would leave it.  These are the building blocks of the
+ * reference's other two TritonGen workloads: LoRA, O = X W + (X A) B (lora_benchmark.py:41-53: X [M,N], W [N,P],
+ * A [N,R], B [R,P], intermediates C = X W, D = X A, E = D B) as  {O, D} = X {W, A};  O = D B + O;  and the gated MLP
+ * (gmlp_benchmark.py:53-64: X [M,K], W1, W2 [K,N], intermediates C1, C1_exp, C2) as  {C1, C2} = X {W1, W2}  followed
+ * by trn_gate_f16.  Same kernels and tile selection as trn_prenorm_qkv_f16 (norm off).  hidden, n_i multiples of 8.
+ */
+int trn_linear_f16(const void* x, int64_t tokens, int64_t hidden, int64_t ldx, int32_t n_mats,
+                   const void* const* w, const int64_t* n, const int64_t* ldw,
+                   void* const* out, const int64_t* ldo, const void* const* addend /* nullable */, void* stream);
+
+/*
+ * Gate of the gated MLP, elementwise over [rows, cols] fp16:  out = sigmoid(c1) * c2  (kind 0)  or
+ * out = c1 * sigmoid(c1) * c2  (kind 1, SiLU).  The reference names the tensors (gmlp_benchmark.py:53-64) and has a
+ * sigmoid operator (NodeType.py:21); the IR that combines them is not in its tree, so both common gates are offered.
+ * cols a multiple of 8; out may alias c1 or c2.
+ */
+int trn_gate_f16(const void* c1, const void* c2, void* out, int64_t rows, int64_t cols,
+                 int64_t ld1, int64_t ld2, int64_t ldo, int32_t kind, void* stream);
+
+/*
  * Measurement aid, no counterpart in the reference: a plain 16-bytes-per-lane streaming copy of `bytes`
  * (a multiple of 16) from src to dst.  bench.py and the profiling recipes run it on a buffer of known size so
  * that HBM byte counters (FETCH_SIZE / WRITE_SIZE) and achieved GB/s of the real kernels can be scaled

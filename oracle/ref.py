@@ -25,7 +25,8 @@ path, so each function is pinned by closed forms, invariants, library routines
 in tests/test_oracle_*.py.  The one convention the reference does not define --
 RoCo's per-key *standard deviation* -- is this build's own (population std over
 the queries that can see the key); it is derived from the two sums the reference
-does define and is marked "parity unpinned" in roco_mean_std below.
+does define and is marked "parity unpinned" in roco_mean_std below.  The same holds for the gate of
+gated_mlp (the reference names the workload's tensors, not the expression): "parity unpinned" there.
 """
 from __future__ import annotations
 
@@ -279,3 +280,29 @@ def harmonic_tail(S: int, power: int = 1) -> torch.Tensor:
     column sums (power 1) and sums of squares (power 2) under uniform attention (Q = 0)."""
     t = 1.0 / torch.arange(1, S + 1, dtype=torch.float64).pow(power)
     return t.flip(0).cumsum(0).flip(0)
+
+
+def lora(X: torch.Tensor, W: torch.Tensor, A: torch.Tensor, B: torch.Tensor) -> torch.Tensor:
+    """O = X W + (X A) B (lora_benchmark.py:41-53; intermediates C = X W, D = X A, E = D B, each an fp16 tensor in
+    the reference's drivers): products in fp32 from fp16 inputs, every intermediate rounded to fp16."""
+    x = X.float()
+    c = (x @ W.float()).half()
+    d = (x @ A.float()).half()
+    e = (d.float() @ B.float()).half()
+    return (c.float() + e.float()).half()
+
+
+def gated_mlp(X: torch.Tensor, W1: torch.Tensor, W2: torch.Tensor, gate: str = "sigmoid") -> torch.Tensor:
+    """O = gate(X W1) * (X W2), gate = sigmoid(c) or c * sigmoid(c) (gmlp_benchmark.py:53-64 names X, W1, W2, O and the
+    intermediates C1, C1_exp, C2; NodeType.py:21 has the sigmoid operator).
+    PARITY UNPINNED beyond its parts: the IR that combines these tensors is not in the reference's tree, so which
+    gate the reference evaluates cannot be read off it; each part is a documented torch primitive."""
+    x = X.float()
+    c1 = (x @ W1.float()).half().float()
+    c2 = (x @ W2.float()).half().float()
+    g = torch.sigmoid(c1)
+    if gate == "silu":
+        g = c1 * g
+    elif gate != "sigmoid":
+        raise ValueError(gate)
+    return (g * c2).half()

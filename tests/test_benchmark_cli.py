@@ -44,3 +44,20 @@ def test_cli_times_every_variant_and_records_failures(variant, tmp_path):
     assert len(data) == 2
     assert data[0]["error"] is None and 0 < data[0]["execution_time_ms"] < 10 and data[0]["tensor_config"]["N"] == 512
     assert data[1]["error"] and math.isinf(data[1]["execution_time_ms"])
+
+
+def test_lora_and_gmlp_shapes_follow_their_drivers():
+    s = benchmark.tensor_shapes({"M": 16, "N": 1024, "P": 512, "R": 64})
+    assert s == {"X": (16, 1024), "W": (1024, 512), "A": (1024, 64), "B": (64, 512), "O": (16, 512)}
+    s = benchmark.tensor_shapes({"M": 16, "N": 2048, "K": 1024})
+    assert s == {"X": (16, 1024), "W1": (1024, 2048), "W2": (1024, 2048), "O": (16, 2048)}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant", benchmark.LINEAR_VARIANTS)
+def test_cli_times_lora_and_gmlp_at_the_reference_shapes(variant, tmp_path):
+    out = tmp_path / "o.json"
+    assert benchmark.main(["--variant", variant, "--output", str(out), "--runs", "5", "--warmup", "2"]) == 0
+    data = json.loads(out.read_text())
+    assert len(data) == len(benchmark.LORA_CONFIGS if variant == "lora" else benchmark.GMLP_CONFIGS)
+    assert all(d["error"] is None and 0 < d["execution_time_ms"] < 10 for d in data)

@@ -98,12 +98,34 @@ CANDIDATES = {
         f"(seq {projections()} {attention(divide_last=False, extra_in_loop=ROCO_STATS)})",
     ],
 }
+LINEAR = {
+    # LoRA (lora_benchmark.py:41-53): X@W + (X@A)@B, fused and in three kernels through the driver's intermediates
+    "lora": [
+        "(ploop 0 P 64 p (store (output O) (+ (* (load (input X) (index fulltile fulltile)) (load (input W) (index fulltile (tile p)))) "
+        "(* (* (load (input X) (index fulltile fulltile)) (load (input A) (index fulltile fulltile))) (load (input B) (index fulltile (tile p))))) (index fulltile (tile p))))",
+        "(seq (ploop 0 R 16 r (store (tensor D) (* (load (input X) (index fulltile fulltile)) (load (input A) (index fulltile (tile r)))) (index fulltile (tile r)))) "
+        "(ploop 0 P 64 p (seq (store (tensor C) (* (load (input X) (index fulltile fulltile)) (load (input W) (index fulltile (tile p)))) (index fulltile (tile p))) "
+        "(store (tensor E) (* (load (tensor D) (index fulltile fulltile)) (load (input B) (index fulltile (tile p)))) (index fulltile (tile p))) "
+        "(store (output O) (+ (load (tensor C) (index fulltile (tile p))) (load (tensor E) (index fulltile (tile p)))) (index fulltile (tile p))))))",
+    ],
+    # gated MLP (gmlp_benchmark.py:53-64), with the sigmoid operator and spelled out with exp
+    "gmlp": [
+        "(ploop 0 N 64 n (store (output O) (x (sigmoid (* (load (input X) (index fulltile fulltile)) (load (input W1) (index fulltile (tile n))))) "
+        "(* (load (input X) (index fulltile fulltile)) (load (input W2) (index fulltile (tile n))))) (index fulltile (tile n))))",
+        "(ploop 0 N 64 n (seq (store (tensor C1) (* (load (input X) (index fulltile fulltile)) (load (input W1) (index fulltile (tile n)))) (index fulltile (tile n))) "
+        "(store (tensor C1_exp) (exp (- 0 (load (tensor C1) (index fulltile (tile n))))) (index fulltile (tile n))) "
+        "(store (tensor C2) (* (load (input X) (index fulltile fulltile)) (load (input W2) (index fulltile (tile n)))) (index fulltile (tile n))) "
+        "(store (output O) (/ (x (load (tensor C1) (index fulltile (tile n))) (load (tensor C2) (index fulltile (tile n)))) "
+        "(+ 1 (load (tensor C1_exp) (index fulltile (tile n))))) (index fulltile (tile n)))))",
+    ],
+}
 UNSUPPORTED = {
-    # LoRA (lora_benchmark.py:41-53): X@W + (X@A)@B
-    "lora": "(ploop 0 N 64 n (store (output O) (+ (* (load (input X) (index fulltile fulltile)) (load (input W) (index fulltile (tile n)))) "
-            "(* (* (load (input X) (index fulltile fulltile)) (load (input A) (index fulltile fulltile))) (load (input B) (index fulltile (tile n))))) (index fulltile (tile n))))",
-    # gated MLP (gmlp_benchmark.py:53-64)
-    "gmlp": "(ploop 0 N 64 n (store (output O2) (x (sigmoid (* (load (input X) (index fulltile fulltile)) (load (input WQ) (index fulltile (tile n))))) "
+    "lora without the adapter": "(ploop 0 P 64 p (store (output O) (+ (* (load (input X) (index fulltile fulltile)) (load (input W) (index fulltile (tile p)))) "
+                                "(+ (load (input A) (index fulltile fulltile)) (load (input B) (index fulltile (tile p))))) (index fulltile (tile p))))".replace("(+ (load (input A)", "(x (load (input A)"),
+    "gated-MLP inputs without a gate": "(ploop 0 N 64 n (store (output O) (x (* (load (input X) (index fulltile fulltile)) (load (input W1) (index fulltile (tile n)))) "
+                                       "(* (load (input X) (index fulltile fulltile)) (load (input W2) (index fulltile (tile n))))) (index fulltile (tile n))))",
+    "unknown inputs": "(ploop 0 N 64 n (store (output O) (* (load (input X) (index fulltile fulltile)) (load (input Wz) (index fulltile (tile n)))) (index fulltile (tile n))))",
+    "sigmoid on attention inputs": "(ploop 0 N 64 n (store (output O2) (x (sigmoid (* (load (input X) (index fulltile fulltile)) (load (input WQ) (index fulltile (tile n))))) "
             "(* (load (input X) (index fulltile fulltile)) (load (input WK) (index fulltile (tile n))))) (index fulltile (tile n))))",
     "projection only": f"(seq {projections()} (ploop 0 H 1 h (store (output O2) (load (tensor Q1) (index fulltile (tile h))) (index fulltile (tile h)))))",
     "no cache append": f"(seq {projections()} {attention()})".replace("(store (input K_cache)", "(store (tensor K_new)"),
@@ -118,6 +140,12 @@ UNSUPPORTED = {
 @pytest.mark.parametrize("variant,index", [(v, i) for v, c in CANDIDATES.items() for i in range(len(c))])
 def test_candidates_are_recognised(variant, index):
     m = ir.recognise(CANDIDATES[variant][index])
+    assert m.variant == variant, m.reason
+
+
+@pytest.mark.parametrize("variant,index", [(v, i) for v, c in LINEAR.items() for i in range(len(c))])
+def test_lora_and_gated_mlp_candidates_are_recognised(variant, index):
+    m = ir.recognise(LINEAR[variant][index])
     assert m.variant == variant, m.reason
 
 
@@ -154,14 +182,14 @@ def test_dataflow_summary_follows_accumulations_and_appends():
 def test_ir_file_reader(tmp_path):
     p = tmp_path / "cands.txt"
     p.write_text("\n".join(["# header", "0: " + CANDIDATES["vanilla"][0].replace("\n", " "), "",
-                            "1: (seq dummydata)", "x7: (seq dummy)", "12:   " + UNSUPPORTED["lora"], "no colon here"]))
+                            "1: (seq dummydata)", "x7: (seq dummy)", "12:   " + UNSUPPORTED["unknown inputs"], "no colon here"]))
     got = ir.read_ir_file(str(p))
     assert [i for i, _ in got] == [0, 12]
     assert ir.recognise(got[0][1]).variant == "vanilla" and not ir.recognise(got[1][1])
 
 
 def ir_file(tmp_path):
-    lines = [f"{i}: " + c for i, c in enumerate([CANDIDATES["vanilla"][0], CANDIDATES["roco"][0], UNSUPPORTED["lora"],
+    lines = [f"{i}: " + c for i, c in enumerate([CANDIDATES["vanilla"][0], CANDIDATES["roco"][0], UNSUPPORTED["unknown inputs"],
                                                   CANDIDATES["keyformer"][1], CANDIDATES["qknorm"][0]])]
     p = tmp_path / "cands.txt"
     p.write_text("\n".join(lines))

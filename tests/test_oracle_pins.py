@@ -251,3 +251,43 @@ def test_decode_append_variants_consistent():
     assert torch.equal(op, o2)
     oq = ref.decode_append_qknorm(X, *W, Kc, Vc, P, D)
     assert oq.shape == (H, M, D) and torch.isfinite(oq.float()).all()
+
+
+def test_lora_closed_forms_and_brute_force():
+    """O = X W + (X A) B: zero adapter, zero base, rank-1 adapter in closed form, fp64 brute force."""
+    g = torch.Generator().manual_seed(7)
+    M, N, P, R = 5, 24, 16, 8
+    X, W = ref.randn_half((M, N), g, 0, 0.5), ref.randn_half((N, P), g, 0, 0.5)
+    A, B = ref.randn_half((N, R), g, 0, 0.5), ref.randn_half((R, P), g, 0, 0.5)
+    zA, zW = torch.zeros_like(A), torch.zeros_like(W)
+    assert torch.equal(ref.lora(X, W, zA, B), (X.float() @ W.float()).half())                 # adapter off
+    assert torch.equal(ref.lora(X, zW, A, B), ((X.float() @ A.float()).half().float() @ B.float()).half())
+    # rank 1: (X a) b^T adds (x_i . a) * b_j
+    a1 = torch.zeros_like(A); a1[:, 0] = A[:, 0]
+    b1 = torch.zeros_like(B); b1[0] = B[0]
+    want = X.double() @ W.double() + torch.outer(X.double() @ a1[:, 0].double(), b1[0].double())
+    assert torch.allclose(ref.lora(X, W, a1, b1).double(), want, rtol=2e-3, atol=2e-3)
+    brute = torch.zeros(M, P, dtype=torch.float64)
+    for i in range(M):
+        for j in range(P):
+            acc = sum(float(X[i, k]) * float(W[k, j]) for k in range(N))
+            acc += sum(sum(float(X[i, k]) * float(A[k, r]) for k in range(N)) * float(B[r, j]) for r in range(R))
+            brute[i, j] = acc
+    assert torch.allclose(ref.lora(X, W, A, B).double(), brute, rtol=4e-3, atol=4e-3)
+    # the identity the fused form rests on: X W + (X A) B = X (W + A B)
+    assert torch.allclose(ref.lora(X, W, A, B).double(), X.double() @ (W.double() + A.double() @ B.double()), rtol=4e-3, atol=4e-3)
+
+
+def test_gated_mlp_parts_and_special_values():
+    """gate(X W1) * (X W2): W1 = 0 gives sigmoid(0) = 1/2 (sigmoid gate) or 0 (SiLU); library sigmoid / silu."""
+    g = torch.Generator().manual_seed(9)
+    X, W1, W2 = ref.randn_half((6, 32), g, 0, 0.5), ref.randn_half((32, 16), g, 0, 0.5), ref.randn_half((32, 16), g, 0, 0.5)
+    c2 = (X.float() @ W2.float()).half().float()
+    assert torch.equal(ref.gated_mlp(X, torch.zeros_like(W1), W2), (0.5 * c2).half())
+    assert torch.equal(ref.gated_mlp(X, torch.zeros_like(W1), W2, "silu"), torch.zeros(6, 16, dtype=torch.float16))
+    c1 = (X.float() @ W1.float()).half().float()
+    assert torch.equal(ref.gated_mlp(X, W1, W2, "silu"), (torch.nn.functional.silu(c1) * c2).half())
+    want = (1.0 / (1.0 + torch.exp(-c1.double()))) * c2.double()
+    assert torch.allclose(ref.gated_mlp(X, W1, W2).double(), want, rtol=1e-3, atol=1e-3)
+    with pytest.raises(ValueError):
+        ref.gated_mlp(X, W1, W2, "relu")

@@ -25,18 +25,31 @@ import sys
 from typing import Dict, List, Optional
 
 VARIANTS = ("vanilla", "prenorm", "qknorm", "keyformer", "roco")
+LINEAR_VARIANTS = ("lora", "gmlp")       # the reference's lora_benchmark.py / gmlp_benchmark.py workloads
+# the shapes those two drivers list (lora_benchmark.py:545-548; gmlp_benchmark.py has the same commented list with
+# the LoRA keys, its class reads M, N, K: the first one is used with K = N)
+LORA_CONFIGS = [{"M": 16, "N": 1024, "P": 512, "R": 64}, {"M": 32, "N": 1024, "P": 512, "R": 64},
+                {"M": 16, "N": 2048, "P": 1024, "R": 128}, {"M": 8, "N": 512, "P": 256, "R": 32}]
+GMLP_CONFIGS = [{"M": 16, "N": 1024, "K": 1024}, {"M": 32, "N": 1024, "K": 1024}, {"M": 16, "N": 2048, "K": 2048}]
 
 
 def tensor_shapes(cfg: Dict[str, int]) -> Dict[str, tuple]:
     """Shapes of the tensors the reference drivers allocate for a configuration
-    (vanilla_llama_benchmark.py:42-77, keyformer_llama_benchmark.py:74-79, roco_llama_benchmark.py:74-75)."""
+    (vanilla_llama_benchmark.py:42-77, keyformer_llama_benchmark.py:74-79, roco_llama_benchmark.py:74-75;
+    lora_benchmark.py:41-53 for {M,N,P,R}, gmlp_benchmark.py:53-64 for {M,N,K})."""
+    if "R" in cfg:
+        M, N, P, R = cfg["M"], cfg["N"], cfg["P"], cfg["R"]
+        return {"X": (M, N), "W": (N, P), "A": (N, R), "B": (R, P), "O": (M, P)}
+    if "K" in cfg:
+        M, N, K = cfg["M"], cfg["N"], cfg["K"]
+        return {"X": (M, K), "W1": (K, N), "W2": (K, N), "O": (M, N)}
     M, N, D, P = cfg["M"], cfg["N"], cfg["D"], cfg["P"]
     H = cfg.get("H", N // D)
     return {"X": (M, N), "WQ": (N, N), "WK": (N, N), "WV": (N, N), "K_cache": (H, P + M, D), "V_cache": (H, P + M, D),
             "O2": (M, N), "noise": (H, M, P + M), "C_out": (H, P + M), "C_out1": (H, P + M), "C_out2": (H, P + M)}
 
 
-OUTPUTS = ("O2", "C_out", "C_out1", "C_out2")
+OUTPUTS = ("O2", "C_out", "C_out1", "C_out2", "O")
 
 
 def make_tensors(cfg: Dict[str, int], names: List[str], device: str = "cuda"):
@@ -49,6 +62,8 @@ def make_tensors(cfg: Dict[str, int], names: List[str], device: str = "cuda"):
             raise ValueError(f"Unknown tensor parameter: {n}")
         if n in OUTPUTS:
             out[n] = torch.zeros(shapes[n], dtype=torch.float16, device=device)
+        elif "K" in cfg:       # the gated-MLP driver draws plain randn (gmlp_benchmark.py:96)
+            out[n] = torch.randn(shapes[n], dtype=torch.float16, device=device)
         else:
             out[n] = torch.randn(shapes[n], dtype=torch.float16, device=device).clamp(-1, 1) * 0.01
     return out
@@ -120,7 +135,8 @@ def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: i
     if not torch.cuda.is_available():
         raise SystemExit("Error: no GPU available; the hand-written kernels have no CPU path")
     if candidates is None:              # no IR file: the one candidate is the hand-written module of `variant`
-        candidates = [(f"trinity_hip/{variant}", f"hand-written gfx950 module ({variant}, decode-append form)", variant, "")]
+        form = "linear" if variant in LINEAR_VARIANTS else "decode-append"
+        candidates = [(f"trinity_hip/{variant}", f"hand-written gfx950 module ({variant}, {form} form)", variant, "")]
     records = []
     for cfg in configs:
         for ir_id, expr, var, reason in candidates:
@@ -128,7 +144,7 @@ def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: i
             try:
                 if var is None:         # the reference records a candidate it cannot compile and carries on (:206-210)
                     raise ValueError(f"unsupported IR: {reason}")
-                module = modules.get(var, "decode", head_dim=cfg["D"])
+                module = modules.get(var, "linear") if var in LINEAR_VARIANTS else modules.get(var, "decode", head_dim=cfg["D"])
                 tensors = make_tensors(cfg, module.TENSOR_PARAMS)
                 rec["execution_time_ms"] = time_module(module, tensors, warmup_runs, benchmark_runs)
             except Exception as e:      # ... and one that fails at run time (:329-332)
@@ -160,7 +176,7 @@ def print_report(records: List[dict], top_k: int) -> None:
 def main(argv=None) -> int:
     from . import configs as shapes
     ap = argparse.ArgumentParser(description="Time the hand-written module of one variant the way the reference's drivers time a candidate")
-    ap.add_argument("--variant", choices=VARIANTS, default="vanilla")
+    ap.add_argument("--variant", choices=VARIANTS + LINEAR_VARIANTS, default="vanilla")
     ap.add_argument("--model", choices=("llama", "falcon"), default="llama",
                     help="built-in decode shape (M=16, P=1024 at the model's widths) when --configs is not given")
     ap.add_argument("--configs", type=str, default=None, help="JSON file: a list of {M, N, D, H, P} tensor configurations")
@@ -177,8 +193,11 @@ def main(argv=None) -> int:
     if a.configs:
         with open(a.configs) as f:
             cfgs = json.load(f)
-        if not isinstance(cfgs, list) or not all(isinstance(c, dict) and {"M", "N", "D", "P"} <= set(c) for c in cfgs):
-            ap.error("--configs: expected a JSON list of objects with M, N, D, P (and optionally H)")
+        ok = lambda c: isinstance(c, dict) and ({"M", "N", "D", "P"} <= set(c) or {"M", "N", "P", "R"} <= set(c) or {"M", "N", "K"} <= set(c))
+        if not isinstance(cfgs, list) or not all(ok(c) for c in cfgs):
+            ap.error("--configs: expected a JSON list of objects with M, N, D, P (and optionally H), or M, N, P, R (LoRA), or M, N, K (gated MLP)")
+    elif a.variant in LINEAR_VARIANTS:
+        cfgs = [dict(c) for c in (LORA_CONFIGS if a.variant == "lora" else GMLP_CONFIGS)]
     else:
         cfgs = [dict(shapes.DECODE_LLAMA if a.model == "llama" else shapes.DECODE_FALCON)]
     cands = candidates_from_ir(a.ir, a.start, None if a.end else a.num) if a.ir else None

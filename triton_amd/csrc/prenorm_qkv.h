@@ -4,9 +4,10 @@
 
 namespace trn {
 
-// One projection: weight [hidden][n] with row pitch ldw, head-split output, and the index of its first
-// column panel in the concatenated [Q | K | V] panel list.
-struct ProjOut { const half_t* w; half_t* out; int64_t ldw, stride_h, stride_s; int n; int tile0; };
+// One projection: weight [hidden][n] with row pitch ldw, head-split output, the index of its first column panel in
+// the concatenated [Q | K | V] panel list, and an optional addend laid out like the output (out = x w + addend; it
+// may be the output itself).  n = 0: no such projection.
+struct ProjOut { const half_t* w; half_t* out; int64_t ldw, stride_h, stride_s; int n; int tile0; const half_t* addend; };
 
 // Panels are GBN (128) or WN (256) columns wide depending on the kernel; n_mtiles counts token tiles likewise.
 struct GemmArgs {
@@ -24,10 +25,13 @@ struct GemmArgs {
 __device__ __forceinline__ int wswz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 // 256 x 256 workgroup tiles, for problems large enough to fill the chip with them (prenorm_qkv_wide.hip).
-int launch_prenorm_qkv_wide(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream);
-int64_t prenorm_qkv_wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv);
+int launch_prenorm_qkv_wide(GemmArgs a, hipStream_t stream);
+int64_t prenorm_qkv_wide_tiles(const GemmArgs& a);
 
 // At most 32 tokens: 64-column panels streamed by four waves that split the contraction (prenorm_qkv_skinny.hip).
-int launch_prenorm_qkv_skinny(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream);
+int launch_prenorm_qkv_skinny(GemmArgs a, hipStream_t stream);
+
+// The 128 x 128 tiling and the choice between the three (prenorm_qkv.hip).
+int launch_projections(GemmArgs a, hipStream_t stream);
 
 }  // namespace trn

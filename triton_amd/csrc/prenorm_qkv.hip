@@ -195,16 +195,59 @@ __global__ __launch_bounds__(256, 2) void prenorm_qkv_kernel(const GemmArgs a) {
         // (LDS operations of one wave execute in order: its reads below see its writes above)
         const int orow = lane >> 3, ocol = (lane & 7) * 8;
         const int n = n0 + wn * 64 + ocol;
-        half_t* obase = P.out + (int64_t)(n / a.head_dim) * P.stride_h + (n % a.head_dim);
+        const int64_t o_off = (int64_t)(n / a.head_dim) * P.stride_h + (n % a.head_dim);
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int tl = j * 8 + orow, t = m0 + wm * 64 + tl;
-            const uint2_t lo = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol]);
-            const uint2_t hi = *reinterpret_cast<const uint2_t*>(&ot[tl * OP + ocol + 4]);
-            if (t < a.T && n < P.n) *reinterpret_cast<uint4_t*>(obase + (int64_t)t * P.stride_s) = uint4_t{lo.x, lo.y, hi.x, hi.y};
+            const half4_t lo = *reinterpret_cast<const half4_t*>(&ot[tl * OP + ocol]);
+            const half4_t hi = *reinterpret_cast<const half4_t*>(&ot[tl * OP + ocol + 4]);
+            half8_t ov = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+            if (t < a.T && n < P.n) {
+                if (P.addend) {
+                    const half8_t ad = *reinterpret_cast<const half8_t*>(P.addend + o_off + (int64_t)t * P.stride_s);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) ov[e] = (half_t)((float)ov[e] + (float)ad[e]);
+                }
+                *reinterpret_cast<half8_t*>(P.out + o_off + (int64_t)t * P.stride_s) = ov;
+            }
         }
     }
 #endif
+}
+
+// The tiling is chosen by problem size.
+int launch_projections(GemmArgs a, hipStream_t stream) {
+    // a handful of tokens (decode): the weight stream is everything
+    if (a.T <= 32) return launch_prenorm_qkv_skinny(a, stream);
+    // 256-token tiles once they alone occupy at least half of the 256 CUs; 128 x 128 tiles below that (short
+    // prefills, where the number of workgroups matters more than the work per staged byte)
+    if (prenorm_qkv_wide_tiles(a) >= 128) return launch_prenorm_qkv_wide(a, stream);
+    a.n_mtiles = (a.T + GBM - 1) / GBM;
+    int t0 = 0;
+    for (int i = 0; i < 3; ++i) { a.p[i].tile0 = t0; t0 += (a.p[i].n + GBN - 1) / GBN; }
+    a.n_panels = t0;
+    a.panels_per_xcd = (a.n_panels + 7) / 8;
+    const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
+    if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
+    hipLaunchKernelGGL(prenorm_qkv_kernel, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+}
+
+// out = act(c1) * c2, elementwise over [rows, cols] fp16 (the gate of a gated MLP); 8 columns per lane
+__global__ __launch_bounds__(256) void gate_kernel(const half_t* c1, const half_t* c2, half_t* out, int64_t rows, int cols,
+                                                   int64_t ld1, int64_t ld2, int64_t ldo, int silu) {
+    const int chunks = cols / 8;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * chunks) return;
+    const int64_t r = i / chunks; const int cc = (int)(i % chunks) * 8;
+    const half8_t u = *reinterpret_cast<const half8_t*>(c1 + r * ld1 + cc), v = *reinterpret_cast<const half8_t*>(c2 + r * ld2 + cc);
+    half8_t o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const float x = (float)u[e], sg = 1.0f / (1.0f + fast_exp2(-x * kLog2e));
+        o[e] = (half_t)((silu ? x * sg : sg) * (float)v[e]);
+    }
+    *reinterpret_cast<half8_t*>(out + r * ldo + cc) = o;
 }
 
 }  // namespace trn
@@ -236,21 +279,52 @@ extern "C" int trn_prenorm_qkv_f16(const void* x, const void* gamma, const void*
     GemmArgs a;
     a.x = (const half_t*)x; a.gamma = (const half_t*)gamma;
     a.T = (int)tokens; a.K = (int)hidden; a.head_dim = (int)head_dim; a.ldx = ldx; a.eps = eps; a.norm = norm ? 1 : 0;
-    a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0};
-    a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, 0};
-    a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, 0};
-    // a handful of tokens (decode): the weight stream is everything
-    if (tokens <= 32) return launch_prenorm_qkv_skinny(a, n_q, n_kv, (hipStream_t)stream);
-    // 256 x 256 tiles once they alone occupy at least half of the 256 CUs; 128 x 128 tiles below that (decode
-    // and short prefills, where the number of workgroups matters more than the work per staged byte)
-    if (prenorm_qkv_wide_tiles(tokens, n_q, n_kv) >= 128) return launch_prenorm_qkv_wide(a, n_q, n_kv, (hipStream_t)stream);
-    a.n_mtiles = (int)((tokens + GBM - 1) / GBM);
-    const int tq = (int)((n_q + GBN - 1) / GBN), tkv = (int)((n_kv + GBN - 1) / GBN);
-    a.p[1].tile0 = tq; a.p[2].tile0 = tq + tkv;
-    a.n_panels = tq + 2 * tkv;
-    a.panels_per_xcd = (a.n_panels + 7) / 8;
-    const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
+    a.p[0] = ProjOut{(const half_t*)wq, (half_t*)q, ldwq, q_stride_h, q_stride_s, (int)n_q, 0, nullptr};
+    a.p[1] = ProjOut{(const half_t*)wk, (half_t*)k, ldwk, k_stride_h, k_stride_s, (int)n_kv, 0, nullptr};
+    a.p[2] = ProjOut{(const half_t*)wv, (half_t*)v, ldwv, v_stride_h, v_stride_s, (int)n_kv, 0, nullptr};
+    return launch_projections(a, (hipStream_t)stream);
+}
+
+extern "C" int trn_linear_f16(const void* x, int64_t tokens, int64_t hidden, int64_t ldx, int32_t n_mats,
+                              const void* const* w, const int64_t* n, const int64_t* ldw, void* const* out,
+                              const int64_t* ldo, const void* const* addend, void* stream) {
+    using namespace trn;
+    if (tokens < 0 || hidden <= 0 || n_mats < 1 || n_mats > 3) return TRN_E_SHAPE;
+    if (!x || !w || !n || !ldw || !out || !ldo) return TRN_E_NULL;
+    if (tokens == 0) return TRN_OK;
+    if (hidden % 8 || tokens > 0x7fffffff || hidden > 0x7fffffff) return TRN_E_SHAPE;
+    if (ldx < hidden) return TRN_E_STRIDE;
+    if (!aligned16(x) || !pitch16(ldx, 2)) return TRN_E_ALIGN;
+    if ((tokens + 256) * ldx * 2 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
+    GemmArgs a;
+    a.x = (const half_t*)x; a.gamma = nullptr;
+    a.T = (int)tokens; a.K = (int)hidden; a.ldx = ldx; a.eps = 0.f; a.norm = 0;
+    // plain row-major outputs [tokens, n_i]: "heads" of 8 columns at a pitch of 8 put column n at offset n
+    a.head_dim = 8;
+    for (int i = 0; i < 3; ++i) a.p[i] = ProjOut{nullptr, nullptr, 0, 0, 0, 0, 0, nullptr};
+    for (int i = 0; i < n_mats; ++i) {
+        if (!w[i] || !out[i]) return TRN_E_NULL;
+        if (n[i] <= 0 || n[i] % 8 || n[i] > 0x7fffffff) return TRN_E_SHAPE;
+        if (ldw[i] < n[i] || ldo[i] < n[i]) return TRN_E_STRIDE;
+        const void* ad = addend ? addend[i] : nullptr;
+        if (!aligned16(w[i]) || !aligned16(out[i]) || (ad && !aligned16(ad)) || !pitch16(ldw[i], 2) || !pitch16(ldo[i], 2)) return TRN_E_ALIGN;
+        if ((hidden + 512) * ldw[i] * 2 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
+        a.p[i] = ProjOut{(const half_t*)w[i], (half_t*)out[i], ldw[i], 8, ldo[i], (int)n[i], 0, (const half_t*)ad};
+    }
+    return launch_projections(a, (hipStream_t)stream);
+}
+
+extern "C" int trn_gate_f16(const void* c1, const void* c2, void* out, int64_t rows, int64_t cols, int64_t ld1,
+                            int64_t ld2, int64_t ldo, int32_t kind, void* stream) {
+    using namespace trn;
+    if (rows < 0 || cols <= 0 || cols % 8 || cols > 0x7fffffff || (kind != 0 && kind != 1)) return TRN_E_SHAPE;
+    if (rows == 0) return TRN_OK;
+    if (!c1 || !c2 || !out) return TRN_E_NULL;
+    if (ld1 < cols || ld2 < cols || ldo < cols) return TRN_E_STRIDE;
+    if (!aligned16(c1) || !aligned16(c2) || !aligned16(out) || !pitch16(ld1, 2) || !pitch16(ld2, 2) || !pitch16(ldo, 2)) return TRN_E_ALIGN;
+    const int64_t work = rows * (cols / 8), grid = (work + 255) / 256;
     if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
-    hipLaunchKernelGGL(prenorm_qkv_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, a);
+    hipLaunchKernelGGL(gate_kernel, dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream, (const half_t*)c1, (const half_t*)c2,
+                       (half_t*)out, rows, (int)cols, ld1, ld2, ldo, kind);
     return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }

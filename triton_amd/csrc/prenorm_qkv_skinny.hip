@@ -179,24 +179,27 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_skinny_kernel(const GemmAr
 #pragma unroll
     for (int q = 0; q < 2; ++q) {
         const int r0 = (wave & 1) * 8 + q * 4;               // four consecutive registers = four consecutive columns
+        const int n = n0 + nb * 32 + 8 * (r0 / 4) + 4 * h;
+        const int64_t o_off = (int64_t)(n / a.head_dim) * P.stride_h + (int64_t)c * P.stride_s + (n % a.head_dim);
+        const bool live = c < a.T && n < P.n;
+        half4_t ad = {(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+        if (live && P.addend) ad = *reinterpret_cast<const half4_t*>(P.addend + o_off);
         half4_t ov;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int idx = ((nb * 16 + r0 + e) * 64 + lane);
             const float v = red01[idx] + red01[32 * 64 + idx] + red23[idx] + red23[32 * 64 + idx];
-            ov[e] = (half_t)(v * rstd);
+            ov[e] = (half_t)((float)(half_t)(v * rstd) + (float)ad[e]);     // the product rounded to fp16 first, as a separate GEMM would leave it
         }
-        const int n = n0 + nb * 32 + 8 * (r0 / 4) + 4 * h;
-        if (c < a.T && n < P.n)
-            *reinterpret_cast<half4_t*>(P.out + (int64_t)(n / a.head_dim) * P.stride_h + (int64_t)c * P.stride_s + (n % a.head_dim)) = ov;
+        if (live) *reinterpret_cast<half4_t*>(P.out + o_off) = ov;
     }
 #endif
 }
 
-int launch_prenorm_qkv_skinny(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream) {
-    const int tq = (int)((n_q + SN - 1) / SN), tkv = (int)((n_kv + SN - 1) / SN);
-    a.p[0].tile0 = 0; a.p[1].tile0 = tq; a.p[2].tile0 = tq + tkv;
-    a.n_panels = tq + 2 * tkv;
+int launch_prenorm_qkv_skinny(GemmArgs a, hipStream_t stream) {
+    int t0 = 0;
+    for (int i = 0; i < 3; ++i) { a.p[i].tile0 = t0; t0 += (a.p[i].n + SN - 1) / SN; }
+    a.n_panels = t0;
     hipLaunchKernelGGL(prenorm_qkv_skinny_kernel, dim3((unsigned)a.n_panels), dim3(256), 0, stream, a);
     return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }

@@ -279,8 +279,10 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
             const int64_t stride_s = pi == 2 ? a.p[2].stride_s : pi == 1 ? a.p[1].stride_s : a.p[0].stride_s;
             const int pn = pi == 2 ? a.p[2].n : pi == 1 ? a.p[1].n : a.p[0].n;
             const int t0 = pi == 2 ? a.p[2].tile0 : pi == 1 ? a.p[1].tile0 : 0;
+            const half_t* addend = pi == 2 ? a.p[2].addend : pi == 1 ? a.p[1].addend : a.p[0].addend;
             const int n = (gg - t0) * WG + (blk & 1) * 32 + ocol;
-            half_t* obase = out + (int64_t)(n / a.head_dim) * stride_h + (n % a.head_dim);
+            const int64_t o_off = (int64_t)(n / a.head_dim) * stride_h + (n % a.head_dim);
+            half_t* obase = out + o_off;
 #pragma unroll
             for (int p = 0; p < 2; ++p) {
 #pragma unroll
@@ -299,8 +301,15 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int tl = j * 16 + orow, t = m0 + wm * 128 + p * 64 + tl;
-                    const uint4_t ov = *reinterpret_cast<const uint4_t*>(&ot[tl * OP + ocol]);
-                    if (t < a.T && n < pn) *reinterpret_cast<uint4_t*>(obase + (int64_t)t * stride_s) = ov;
+                    half8_t ov = *reinterpret_cast<const half8_t*>(&ot[tl * OP + ocol]);
+                    if (t < a.T && n < pn) {
+                        if (addend) {
+                            const half8_t ad = *reinterpret_cast<const half8_t*>(addend + o_off + (int64_t)t * stride_s);
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) ov[e] = (half_t)((float)ov[e] + (float)ad[e]);
+                        }
+                        *reinterpret_cast<half8_t*>(obase + (int64_t)t * stride_s) = ov;
+                    }
                 }
             }
         }
@@ -309,24 +318,25 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
 }
 
 // Tiles of nb 64-column groups over the group axis [Q | K | V], each output padded to whole groups.
-static int64_t wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv, int nb) {
-    const int64_t groups = (n_q + WG - 1) / WG + 2 * ((n_kv + WG - 1) / WG);
-    return ((tokens + WM - 1) / WM) * ((groups + nb - 1) / nb);
+static int64_t wide_tiles(const GemmArgs& a, int nb) {
+    int64_t groups = 0;
+    for (int i = 0; i < 3; ++i) groups += (a.p[i].n + WG - 1) / WG;
+    return (((int64_t)a.T + WM - 1) / WM) * ((groups + nb - 1) / nb);
 }
 
 // 192-column tiles when they keep the chip busier: the time is (rounds of 256 workgroups) x (work per tile), and a
 // 192-wide tile does 3/4 of the work of a 256-wide one at slightly lower efficiency (fewer MFMAs per operand read).
-static bool narrow_is_better(int64_t tokens, int64_t n_q, int64_t n_kv) {
-    const int64_t r4 = (wide_tiles(tokens, n_q, n_kv, 4) + 255) / 256, r3 = (wide_tiles(tokens, n_q, n_kv, 3) + 255) / 256;
+static bool narrow_is_better(const GemmArgs& a) {
+    const int64_t r4 = (wide_tiles(a, 4) + 255) / 256, r3 = (wide_tiles(a, 3) + 255) / 256;
     return r3 * 3 * 100 < r4 * 4 * 95;
 }
 
-int launch_prenorm_qkv_wide(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t stream) {
-    const int nb = narrow_is_better(a.T, n_q, n_kv) ? 3 : 4;
+int launch_prenorm_qkv_wide(GemmArgs a, hipStream_t stream) {
+    const int nb = narrow_is_better(a) ? 3 : 4;
     a.n_mtiles = (a.T + WM - 1) / WM;
-    const int gq = (int)((n_q + WG - 1) / WG), gkv = (int)((n_kv + WG - 1) / WG);
-    a.p[0].tile0 = 0; a.p[1].tile0 = gq; a.p[2].tile0 = gq + gkv;      // first group of each output
-    a.n_panels = (gq + 2 * gkv + nb - 1) / nb;
+    int g0 = 0;
+    for (int i = 0; i < 3; ++i) { a.p[i].tile0 = g0; g0 += (a.p[i].n + WG - 1) / WG; }      // first group of each output
+    a.n_panels = (g0 + nb - 1) / nb;
     a.panels_per_xcd = (a.n_panels + 7) / 8;
     const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
     if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
@@ -336,6 +346,6 @@ int launch_prenorm_qkv_wide(GemmArgs a, int64_t n_q, int64_t n_kv, hipStream_t s
 }
 
 // Workgroups the 256-column tiling would launch (useful ones, not counting the padding of the XCD mapping).
-int64_t prenorm_qkv_wide_tiles(int64_t tokens, int64_t n_q, int64_t n_kv) { return wide_tiles(tokens, n_q, n_kv, 4); }
+int64_t prenorm_qkv_wide_tiles(const GemmArgs& a) { return wide_tiles(a, 4); }
 
 }  // namespace trn

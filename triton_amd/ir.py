@@ -229,8 +229,29 @@ ATTENTION_INPUTS = frozenset({"X", "WQ", "WK", "WV", "K_cache", "V_cache"})
 FINAL_OUTPUTS = ("O2", "C_out", "C_out1", "C_out2")
 
 
+def _recognise_linear(df: Dataflow) -> Optional[Match]:
+    """The reference's two other workloads, told apart from attention by their input names: LoRA reads X, W, A, B
+    (lora_benchmark.py:41-53) and writes O = X W + (X A) B; the gated MLP reads X, W1, W2 (gmlp_benchmark.py:53-64)
+    and writes O = gate(X W1) * (X W2)."""
+    o = df.stored.get("O")
+    if df.inputs == {"X", "W", "A", "B"}:
+        if o is None or o.srcs != df.inputs:
+            return Match(None, "LoRA inputs, but O does not depend on all of X, W, A, B")
+        if o.ops != {"matmul", "add"}:
+            return Match(None, f"LoRA inputs, but O is not a sum of matrix products (operators {sorted(o.ops)})")
+        return Match("lora", "O sums the base product and the two-step adapter product")
+    if df.inputs == {"X", "W1", "W2"}:
+        if o is None or o.srcs != df.inputs:
+            return Match(None, "gated-MLP inputs, but O does not depend on all of X, W1, W2")
+        if not {"matmul", "mul"} <= o.ops or not ({"sigmoid"} <= o.ops or {"exp", "div"} <= o.ops):
+            return Match(None, f"gated-MLP inputs, but O is not a gated product (operators {sorted(o.ops)})")
+        return Match("gmlp", "the product with W1, through a sigmoid gate, multiplies the product with W2")
+    return None
+
+
 def recognise(ir: Union[str, Node]) -> Match:
-    """Which of the five decode-append workloads (ref_rms.py:45-83 Vanila, :101-127 PreNorm, :147-179 KeyFormer,
+    """Which workload an IR candidate computes: LoRA or the gated MLP (by their input names, see above), or one of
+    the five decode-append attention workloads (ref_rms.py:45-83 Vanila, :101-127 PreNorm, :147-179 KeyFormer,
     :197-231 QKNorm, :249-280 RoCo) an IR candidate computes, by dataflow:
 
     * O2 derives from X, WQ, WK, WV and both caches through matmul, exp and a division (softmax attention);
@@ -244,6 +265,9 @@ def recognise(ir: Union[str, Node]) -> Match:
         df = analyse(tree)
     except (ValueError, IndexError, RecursionError) as e:
         return Match(None, f"cannot parse: {e}")
+    linear = _recognise_linear(df)
+    if linear is not None:
+        return linear
     extra = df.inputs - ATTENTION_INPUTS - {"noise"}
     if extra:
         return Match(None, f"reads inputs no attention variant has: {sorted(extra)}")

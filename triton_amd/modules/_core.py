@@ -342,17 +342,59 @@ class DecodeRoCo(_DecodeAppend):
         _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
 
 
+class LoRA(FusedModule):
+    """O = X W + (X A) B  (lora_benchmark.py:41-53: X [M,N], W [N,P], A [N,R], B [R,P], O [M,P]; the driver's
+    intermediates C = X W, D = X A, E = D B stay inside: D is a workspace, C and E never leave the kernels).
+    Two launches: {O, D} = X {W, A}, then O = D B + O."""
+    TENSOR_PARAMS = ["A", "B", "O", "W", "X"]
+
+    def _run(self, A, B, O, W, X):
+        M, N = X.shape
+        R, P = B.shape
+        if W.shape != (N, P) or A.shape != (N, R) or O.shape != (M, P):
+            raise ValueError(f"inconsistent shapes: X {tuple(X.shape)}, W {tuple(W.shape)}, A {tuple(A.shape)}, B {tuple(B.shape)}, O {tuple(O.shape)}")
+        d = self._workspace("D", (M, R), X.dtype, X.device)
+        ops.linear(X, [W, A], [O, d])
+        ops.linear(d, [B], [O], [O])
+
+
+class GatedMLP(FusedModule):
+    """O = gate(X W1) * (X W2)  (gmlp_benchmark.py:53-64: X [M,K], W1, W2 [K,N], O [M,N]; intermediates C1, C1_exp,
+    C2).  gate = 'sigmoid' (sigmoid(C1)) or 'silu' (C1 sigmoid(C1)): the reference names the tensors and has a sigmoid
+    operator, but the IR that combines them is not in its tree.  One GEMM launch for both products, one for the gate."""
+    TENSOR_PARAMS = ["O", "W1", "W2", "X"]
+
+    def __init__(self, gate: str = "sigmoid"):
+        super().__init__()
+        if gate not in ("sigmoid", "silu"):
+            raise ValueError("gate: expected 'sigmoid' or 'silu'")
+        self.gate = gate
+
+    def _run(self, O, W1, W2, X):
+        M, K = X.shape
+        if W1.shape[0] != K or W1.shape != W2.shape or O.shape != (M, W1.shape[1]):
+            raise ValueError(f"inconsistent shapes: X {tuple(X.shape)}, W1 {tuple(W1.shape)}, W2 {tuple(W2.shape)}, O {tuple(O.shape)}")
+        c2 = self._workspace("C2", tuple(O.shape), X.dtype, X.device)
+        ops.linear(X, [W1, W2], [O, c2])            # C1 lands in O and is gated in place
+        ops.gate(O, c2, O, self.gate)
+
+
 PREFILL = {"rms": RMSNorm, "vanilla": Attention, "prenorm": PreNormBlock, "qknorm": QKNormAttention,
            "keyformer": KeyFormerAttention, "roco": RoCoAttention}
 DECODE = {"vanilla": DecodeVanilla, "prenorm": lambda **kw: DecodeVanilla(prenorm=True, **kw),
           "qknorm": DecodeQKNorm, "keyformer": DecodeKeyFormer, "roco": DecodeRoCo}
 
 
+LINEAR = {"lora": LoRA, "gmlp": GatedMLP}
+
+
 def get(variant: str, form: str = "prefill", **consts) -> FusedModule:
-    """Module for `variant` in {'rms','vanilla','prenorm','qknorm','keyformer','roco'}.
+    """Module for `variant` in {'rms','vanilla','prenorm','qknorm','keyformer','roco'} (attention forms) or
+    {'lora','gmlp'} (form='linear').
     form='prefill': Q/K/V (or X and weights) given, causal, 1/sqrt(D) scale by default.
-    form='decode' : the reference's decode-append problem (needs head_dim=...)."""
-    table = PREFILL if form == "prefill" else DECODE if form == "decode" else None
+    form='decode' : the reference's decode-append problem (needs head_dim=...).
+    form='linear' : the reference's LoRA and gated-MLP workloads."""
+    table = {"prefill": PREFILL, "decode": DECODE, "linear": LINEAR}.get(form)
     if table is None or variant not in table:
         raise KeyError(f"no module for variant={variant!r} form={form!r}")
     return table[variant](**consts)

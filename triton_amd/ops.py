@@ -186,6 +186,43 @@ def prenorm_qkv(x: torch.Tensor, gamma: Optional[torch.Tensor], wq, wk, wv, q_ou
     _lib.check("trn_prenorm_qkv_f16", st)
 
 
+def linear(x: torch.Tensor, weights, outs, addends=None) -> None:
+    """outs[i] = x @ weights[i] (+ addends[i]) for up to three weight matrices sharing x.  x [T, hidden]; weights[i]
+    [hidden, n_i]; outs[i] / addends[i] [T, n_i]; rows may be strided, innermost stride 1; an addend may be its out."""
+    _dev_half(x, "x")
+    _need(x.dim() == 2, "x: expected [tokens, hidden]")
+    T, K = x.shape
+    k = len(weights)
+    _need(1 <= k <= 3 and len(outs) == k and (addends is None or len(addends) == k), "expected 1-3 weights with as many outputs")
+    adds = list(addends) if addends is not None else [None] * k
+    for i, (w, o, ad) in enumerate(zip(weights, outs, adds)):
+        _dev_half(w, f"weights[{i}]"); _dev_half(o, f"outs[{i}]")
+        _need(w.dim() == 2 and w.shape[0] == K, f"weights[{i}]: expected [hidden={K}, n], got {tuple(w.shape)}")
+        _need(tuple(o.shape) == (T, w.shape[1]), f"outs[{i}]: expected [{T}, {w.shape[1]}], got {tuple(o.shape)}")
+        if ad is not None:
+            _dev_half(ad, f"addends[{i}]")
+            _need(tuple(ad.shape) == tuple(o.shape) and ad.stride() == o.stride(), f"addends[{i}]: expected the shape and strides of outs[{i}]")
+    vps = lambda ts: (C.c_void_p * k)(*[_ptr(t) for t in ts])
+    i64 = lambda vs: (C.c_int64 * k)(*vs)
+    lib = _lib.load()
+    st = lib.trn_linear_f16(_ptr(x), T, K, x.stride(0), k, vps(weights), i64([w.shape[1] for w in weights]),
+                            i64([w.stride(0) for w in weights]), vps(outs), i64([o.stride(0) for o in outs]),
+                            vps(adds), _stream(x))
+    _lib.check("trn_linear_f16", st)
+
+
+def gate(c1: torch.Tensor, c2: torch.Tensor, out: torch.Tensor, kind: str = "sigmoid") -> None:
+    """out = sigmoid(c1) * c2 ("sigmoid") or c1 * sigmoid(c1) * c2 ("silu"), elementwise over [rows, cols] fp16."""
+    _need(kind in ("sigmoid", "silu"), "kind: expected 'sigmoid' or 'silu'")
+    for t, n in ((c1, "c1"), (c2, "c2"), (out, "out")):
+        _dev_half(t, n)
+        _need(t.dim() == 2 and tuple(t.shape) == tuple(c1.shape), f"{n}: expected [rows, cols] like c1")
+    lib = _lib.load()
+    st = lib.trn_gate_f16(_ptr(c1), _ptr(c2), _ptr(out), c1.shape[0], c1.shape[1], c1.stride(0), c2.stride(0),
+                          out.stride(0), 1 if kind == "silu" else 0, _stream(c1))
+    _lib.check("trn_gate_f16", st)
+
+
 def calibration_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     """dst <- src with the library's plain streaming copy kernel (measurement yardstick)."""
     _need(src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous(), "expected contiguous GPU tensors")
