@@ -1,4 +1,4 @@
-"""Writes tests/golden/kat_small.npz: small known-answer vectors for the six operators.
+"""Writes tests/golden/kat_small.npz: small known-answer vectors for the six operators, LoRA and the gated MLP.
 
 The reference ships no golden vectors for this path, so these come from the fp64 loop-level definitions in
 oracle/brute.py (written from the mathematics, independently of oracle/ref.py's tensor expressions) on seeded fp16
@@ -57,6 +57,16 @@ def main():
     xn = brute.rmsnorm(x, g.astype(np.float64), 1e-5)
     out.update(prj_x=x, prj_gamma=g, prj_wq=wq, prj_wk=wk, prj_wv=wv, prj_eps=np.float32(1e-5),
                prj_q=xn @ wq.astype(np.float64), prj_k=xn @ wk.astype(np.float64), prj_v=xn @ wv.astype(np.float64))
+    # LoRA (lora_benchmark.py:41-53) and the two gates of the gated MLP (gmlp_benchmark.py:53-64), in fp64 from the
+    # definitions (drawn last, so that the vectors above stay as they were)
+    x = h16(rng, (5, 64), 0.5); w = h16(rng, (64, 48), 0.05); la = h16(rng, (64, 8), 0.05); lb = h16(rng, (8, 48), 0.2)
+    x64 = x.astype(np.float64)
+    out.update(lora_x=x, lora_w=w, lora_a=la, lora_b=lb,
+               lora_o=x64 @ w.astype(np.float64) + (x64 @ la.astype(np.float64)) @ lb.astype(np.float64))
+    w1 = h16(rng, (64, 40), 0.1); w2 = h16(rng, (64, 40), 0.1)
+    c1 = x64 @ w1.astype(np.float64); c2 = x64 @ w2.astype(np.float64)
+    sg = 1.0 / (1.0 + np.exp(-c1))
+    out.update(gmlp_x=x, gmlp_w1=w1, gmlp_w2=w2, gmlp_o_sigmoid=sg * c2, gmlp_o_silu=c1 * sg * c2)
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "kat_small.npz")
     np.savez_compressed(path, **{n: (a if a.dtype in (np.float16, np.float32) else np.asarray(a, np.float32))
                                  for n, a in ((n, np.asarray(a)) for n, a in out.items())})

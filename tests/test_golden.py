@@ -84,6 +84,27 @@ def test_hip_attention_scores_kat(case, causal):
         close(o[0], T("gqa_o"), 2e-2, 1e-2)
 
 
+def test_oracle_lora_and_gated_mlp_kat():
+    close(ref.lora(T("lora_x"), T("lora_w"), T("lora_a"), T("lora_b")), T("lora_o"), 2e-3, 2e-3)
+    close(ref.gated_mlp(T("gmlp_x"), T("gmlp_w1"), T("gmlp_w2"), "sigmoid"), T("gmlp_o_sigmoid"), 2e-3, 2e-3)
+    close(ref.gated_mlp(T("gmlp_x"), T("gmlp_w1"), T("gmlp_w2"), "silu"), T("gmlp_o_silu"), 2e-3, 2e-3)
+
+
+@pytest.mark.gpu
+def test_hip_lora_and_gated_mlp_kat():
+    from triton_amd import modules
+    t = dict(X=T("lora_x").cuda(), W=T("lora_w").cuda(), A=T("lora_a").cuda(), B=T("lora_b").cuda())
+    t["O"] = torch.zeros(5, 48, dtype=torch.float16, device="cuda")
+    mod = modules.get("lora", "linear")
+    mod.forward(*[t[n] for n in mod.TENSOR_PARAMS])
+    close(t["O"], T("lora_o"), 2e-3, 1e-2)
+    for gate in ("sigmoid", "silu"):
+        t = dict(X=T("gmlp_x").cuda(), W1=T("gmlp_w1").cuda(), W2=T("gmlp_w2").cuda(), O=torch.zeros(5, 40, dtype=torch.float16, device="cuda"))
+        mod = modules.get("gmlp", "linear", gate=gate)
+        mod.forward(*[t[n] for n in mod.TENSOR_PARAMS])
+        close(t["O"], T("gmlp_o_" + gate), 2e-3, 1e-2)
+
+
 @pytest.mark.gpu
 def test_hip_qknorm_and_projection_kat():
     from triton_amd import modules, ops
