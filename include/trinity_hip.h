@@ -140,6 +140,20 @@ int trn_attn_colstats_f16(const trn_attn_desc* desc, const void* q, const void* 
                           float* out_sum, float* out_sumsq, void* stream);
 
 /*
+ * trn_attn_fwd_f16 and trn_attn_colstats_f16 in one call: the attention output plus the per-key statistics of its
+ * probabilities -- of the perturbed probabilities when noise is given -- i.e. what one forward of the reference's
+ * KeyFormer (ref_rms.py:147-179, C_out of keyformer_llama_benchmark.py:79) or RoCo (ref_rms.py:249-280) computes.
+ * With at most 32 queries per head (the reference's decode-append problem) the statistics are a second sweep over
+ * the keys inside the attention kernel -- one launch; otherwise the two kernels are launched one after the other,
+ * and lse (lse_pert with noise) is required as the buffer that carries the row normalisers between them.
+ * q_norm is not supported here.  out_sum / out_sumsq as in trn_attn_colstats_f16 (one of them may be NULL).
+ */
+int trn_attn_fwd_stats_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                           void* o, float* lse, const void* gamma_q,
+                           const float* noise, float* lse_pert,
+                           float* out_sum, float* out_sumsq, void* stream);
+
+/*
  * Fused RMSNorm + Q/K/V projection:  Xn = RMSNorm(X; gamma, eps);  Q = Xn Wq, K = Xn Wk,
  * V = Xn Wv  (X @ W, W is [hidden, n_out] row-major -- ref_rms.py:105-107, and the per-head
  * column slices of convert_eval_rms.py:132-138).  The row mean-square is reduced inside the

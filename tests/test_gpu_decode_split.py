@@ -148,7 +148,8 @@ def test_split_keys_under_graph_replay():
 
 
 def test_decode_modules_split_path_matches_reference_classes():
-    """The decode-append modules at a shape where the attention splits its keys (8 heads, 1040 keys)."""
+    """The decode-append modules at a shape where the attention splits its keys (8 heads, 1040 keys); RoCo asks for
+    the key statistics, which are a second sweep of the one workgroup per head, so it is not split."""
     from triton_amd import modules
     M, N, D, P = 16, 1024, 128, 1024
     H = N // D
@@ -166,8 +167,8 @@ def test_decode_modules_split_path_matches_reference_classes():
         for _ in range(2):
             mod.forward(*[t[n] for n in mod.TENSOR_PARAMS])
         torch.cuda.synchronize()
-        assert any(k[0] == "attn_ws" for k in mod._ws), "expected the split path"
         if variant == "vanilla":
+            assert any(k[0] == "attn_ws" for k in mod._ws), "expected the split path"
             want = ref.decode_append_vanilla(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)
             close(t["O2"], ref.flatten_token_major(want))
         else:

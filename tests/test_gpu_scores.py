@@ -83,3 +83,62 @@ def test_colstats_deterministic():
     _, a1, a2 = run_roco(q, k, v, 0.088, True)
     _, b1, b2 = run_roco(q, k, v, 0.088, True)
     assert torch.equal(a1, b1) and torch.equal(a2, b2)
+
+
+# ---- trn_attn_fwd_stats_f16: attention + statistics in one call (one launch with at most 32 queries per head)
+FUSED = [(1, 4, 4, 16, 1040, 128, False), (1, 4, 2, 16, 1040, 128, True), (2, 6, 1, 7, 333, 64, True),
+         (1, 3, 3, 32, 32, 128, True), (1, 2, 2, 1, 100, 64, False), (1, 71, 1, 16, 1040, 64, False),
+         (1, 4, 2, 130, 259, 128, True)]                     # more than 32 queries: two launches inside the call
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", FUSED)
+def test_fused_attention_and_roco_statistics(B, Hq, Hkv, Sq, Skv, D, causal):
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=11)
+    scale = D ** -0.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda")
+    s1 = torch.full((B, Hq, Skv), -1.0, device="cuda"); s2 = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention_with_stats(qd, kd, vd, o, scale, causal, s1, s2, lse=lse)
+    torch.cuda.synchronize()
+    wo, w1, w2 = ref.roco(q, k, v, scale, causal)
+    close_scores(s1, w1); close_scores(s2, w2)
+    assert (o.float().cpu() - wo.float()).abs().max() < 2e-2
+    assert torch.allclose(s1.sum(-1).cpu(), torch.full((B, Hq), float(Sq)), rtol=1e-4)
+    # the same numbers as the two separate calls (within summation order)
+    o2, t1, t2 = run_roco(q, k, v, scale, causal)
+    close_scores(s1, t1.cpu(), rtol=1e-4); close_scores(s2, t2.cpu(), rtol=1e-4)
+    # only one of the two statistics
+    s1b = torch.full_like(s1, -1.0)
+    ops.attention_with_stats(qd, kd, vd, o, scale, causal, s1b, None, lse=lse)
+    torch.cuda.synchronize()
+    assert torch.equal(s1b, s1)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,tau", [(1, 4, 4, 16, 1040, 128, False, 1.5), (2, 4, 2, 9, 700, 128, True, 1.5),
+                                                          (1, 3, 1, 32, 100, 64, True, 1.0), (1, 2, 1, 130, 260, 64, True, 1.0)])
+def test_fused_attention_and_keyformer_scores(B, Hq, Hkv, Sq, Skv, D, causal, tau):
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=7)
+    noise = ref.gumbel_noise((B, Hq, Sq, Skv), 1234)
+    scale = D ** -0.5
+    o = torch.zeros_like(q).cuda(); lsep = torch.zeros(B, Hq, Sq, device="cuda")
+    score = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention_with_stats(q.cuda(), k.cuda(), v.cuda(), o, scale, causal, score, None, noise=noise.cuda(), tau=tau, lse_pert=lsep)
+    torch.cuda.synchronize()
+    wo, wscore = ref.keyformer(q, k, v, noise, scale, tau, causal)
+    close_scores(score, wscore)
+    assert (o.float().cpu() - wo.float()).abs().max() < 2e-2
+    assert torch.allclose(score.sum(-1).cpu(), torch.full((B, Hq), float(Sq)), rtol=1e-4)
+
+
+def test_fused_statistics_argument_rules():
+    from triton_amd import ops, _lib
+    q, k, v = make(1, 2, 2, 64, 64, 64)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); s1 = torch.zeros(1, 2, 64, device="cuda")
+    with pytest.raises(_lib.TrnError) as e:          # more than 32 queries and no buffer for the row normalisers
+        ops.attention_with_stats(qd, kd, vd, o, 0.125, True, s1)
+    assert e.value.status_name == "TRN_E_NULL"
+    with pytest.raises(ValueError):
+        ops.attention_with_stats(qd, kd, vd, o, 0.125, True, None, None)

@@ -16,6 +16,9 @@ struct AttnArgs {
     // decode kernel only: keys split over n_split workgroups per head, partial results and arrival counters in ws
     int n_split;
     float* ws;
+    // decode kernel only, one workgroup per head: per-key sums (and sums of squares) of the probabilities -- of the
+    // perturbed ones when noise is given -- from a second sweep over the keys once the row normalisers are final
+    float* col_sum; float* col_sumsq;
 };
 
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).

@@ -351,6 +351,67 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             if (dg == 1 && q < a.Sq) a.lse_pert[(int64_t)bh * a.Sq + q] = (ms2 + fast_log2(L2)) * kLn2;
         }
     }
+    // ---- column statistics (KeyFormer key scores, RoCo sums): a second sweep over this head's keys now that the
+    // row normalisers are final.  The score block is formed the other way round, S[query][key] -- the same two
+    // register operands with their roles swapped -- so that a lane owns one KEY and holds 16 of the 32 queries: the
+    // sum over queries is in-lane plus one exchange with lane^32, and a block's 32 sums are one 128-byte store.
+    // (Only with one workgroup per head: the launcher does not split the keys when these outputs are asked for.)
+    if (a.col_sum || a.col_sumsq) {
+        __syncthreads();                                   // every thread has read the merge arrays
+        if (dg == 0) st_l[0][q] = NOISE ? ms2 + fast_log2(L2) : mstar + fast_log2(L);     // log2 domain
+        __syncthreads();
+        float lq[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) lq[r] = st_l[0][8 * (r / 4) + 4 * h + (r % 4)];
+        const float cs = NOISE ? a.c2 : a.c1;
+        // noise of the lane's key for its 16 queries: 16 dwords from 16 rows, consecutive keys in consecutive lanes
+        float gs0[NOISE ? 16 : 1], gs1[NOISE ? 16 : 1];
+        auto fetch_noise_col = [&](int blk, float (&g)[NOISE ? 16 : 1]) __attribute__((always_inline)) {
+            if constexpr (NOISE) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int qr = 8 * (r / 4) + 4 * h + (r % 4);
+                    g[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                        nrs, (int)((qr * a.ns + c) * 4), blk * 128, 0));
+                }
+            }
+        };
+        // (one block ahead is enough: with one workgroup per head the sweep runs at what a single CU can pull from
+        // L2, about 55 GB/s; requesting two blocks ahead measured the same)
+        auto sweep = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], float (&gc)[NOISE ? 16 : 1], float (&gn)[NOISE ? 16 : 1])
+                         __attribute__((always_inline)) {
+            const int blk = blk0 + wave + it * DNW, key = blk * 32 + c;
+            fetch_k(blk + DNW, kn);
+            fetch_noise_col(blk + DNW, gn);
+            float16_t s;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < NS; ++ks) s = mfma32(qB[ks], kc[ks], s);
+            float x = 0.f, y = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int qr = 8 * (r / 4) + 4 * h + (r % 4);
+                float t = __builtin_fmaf(s[r], cs, -lq[r]);
+                if constexpr (NOISE) t = __builtin_fmaf(gc[r], a.c3, t);
+                const bool ok = key < a.Skv && qr < a.Sq && (!a.causal || key <= qr + off);
+                const float p = ok ? fast_exp2(t) : 0.f;
+                x += p;
+                y = __builtin_fmaf(p, p, y);
+            }
+            x = half_sum(x); y = half_sum(y);
+            if (h == 0 && key < a.Skv) {
+                if (a.col_sum) a.col_sum[(int64_t)bh * a.Skv + key] = x;
+                if (a.col_sumsq) a.col_sumsq[(int64_t)bh * a.Skv + key] = y;
+            }
+        };
+        fetch_k(blk0 + wave, ka0);
+        fetch_noise_col(blk0 + wave, gs0);
+        for (int it = 0; it < nmine; it += 2) {
+            sweep(it, ka0, ka1, gs0, gs1);
+            if (it + 1 < nmine) sweep(it + 1, ka1, ka0, gs1, gs0);
+        }
+    }
 #endif
 }
 
@@ -378,7 +439,7 @@ int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     a.n_split = 1; a.ws = nullptr;
     const int64_t need = attn_decode_workspace_bytes(a.B, a.Hq, a.Sq, a.Skv, head_dim);
-    if (workspace && need > 0 && workspace_bytes >= need) {
+    if (workspace && need > 0 && workspace_bytes >= need && !a.col_sum && !a.col_sumsq) {
         a.n_split = decode_splits(a.B, a.Hq, a.Skv, head_dim);
         a.ws = static_cast<float*>(workspace);
     }

@@ -421,10 +421,41 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     return trn_attn_fwd_ws_f16(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, stream);
 }
 
+namespace trn {
+static int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
+                        const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
+                        int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream);
+}
+
 extern "C" int trn_attn_fwd_ws_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
                                    float* lse, const void* gamma_q, const float* noise, float* lse_pert,
                                    void* workspace, int64_t workspace_bytes, void* stream) {
+    return trn::attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, workspace, workspace_bytes, nullptr, nullptr, stream);
+}
+
+extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, const void* k, const float* lse,
+                                     const float* noise, float* out_sum, float* out_sumsq, void* stream);
+
+extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                      float* lse, const void* gamma_q, const float* noise, float* lse_pert,
+                                      float* out_sum, float* out_sumsq, void* stream) {
     using namespace trn;
+    if (!d) return TRN_E_NULL;
+    if (!out_sum && !out_sumsq) return TRN_E_NULL;
+    if (d->q_norm) return TRN_E_UNSUPPORTED;     // the statistics pass takes the queries as given
+    // a handful of queries per head: the statistics are a second sweep inside the same kernel
+    if (d->seq_q <= 32) return attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, out_sum, out_sumsq, stream);
+    // otherwise two launches; the second needs the first one's row normalisers
+    float* rows = noise ? lse_pert : lse;
+    if (!rows) return TRN_E_NULL;
+    const int st = attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, nullptr, nullptr, stream);
+    if (st != TRN_OK) return st;
+    return trn_attn_colstats_f16(d, q, k, rows, noise, out_sum, out_sumsq, stream);
+}
+
+static int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
+                             const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
+                             int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream) {
     if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;
     if (!d || !q || !k || !v || !o) return TRN_E_NULL;
     if (noise && !lse_pert) return TRN_E_NULL;
@@ -455,6 +486,7 @@ extern "C" int trn_attn_fwd_ws_f16(const trn_attn_desc* d, const void* q, const 
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
+    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
     if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)

@@ -319,8 +319,9 @@ class DecodeKeyFormer(_DecodeAppend):
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
         score = C_out.view(1, H, PM) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
             self._workspace("score32", (1, H, PM), torch.float32, X.device)
-        self._attend(q, K_cache, V_cache, O2, noise=n4, tau=self.tau, lse_pert=lsep)
-        ops.attention_colstats(q[None], K_cache[None], lsep, self.scale, self.causal, score, None, noise=n4, tau=self.tau)
+        # one launch up to 32 new tokens (the key scores are a second sweep inside the attention kernel), two beyond
+        ops.attention_with_stats(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
+                                 score, None, noise=n4, tau=self.tau, lse_pert=lsep)
         _store_scores(C_out, score)
 
 
@@ -337,8 +338,8 @@ class DecodeRoCo(_DecodeAppend):
         for i, c in enumerate((C_out1, C_out2)):
             outs.append(c.view(1, H, PM) if c.dtype == torch.float32 and c.is_contiguous() else
                         self._workspace(f"stat32_{i}", (1, H, PM), torch.float32, X.device))
-        self._attend(q, K_cache, V_cache, O2, lse=lse)
-        ops.attention_colstats(q[None], K_cache[None], lse, self.scale, self.causal, outs[0], outs[1])
+        ops.attention_with_stats(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
+                                 outs[0], outs[1], lse=lse)
         _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
 
 

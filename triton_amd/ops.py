@@ -157,6 +157,27 @@ def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[
     _lib.check("trn_attn_colstats_f16", st)
 
 
+def attention_with_stats(q, k, v, o, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
+                         out_sumsq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                         noise: Optional[torch.Tensor] = None, tau: float = 1.0,
+                         lse_pert: Optional[torch.Tensor] = None) -> None:
+    """`attention` and `attention_colstats` in one call (one launch with at most 32 queries per head): o, and the
+    column sums / sums of squares of the probabilities -- of the perturbed ones when noise is given.  With more than
+    32 queries lse (lse_pert with noise) must be given: it carries the row normalisers between the two kernels."""
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, noise, tau)
+    B, Hq, Sq, _ = q.shape
+    Skv = k.shape[2]
+    _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq))
+    _row_stat(out_sum, "out_sum", (B, Hq, Skv)); _row_stat(out_sumsq, "out_sumsq", (B, Hq, Skv))
+    _need(out_sum is not None or out_sumsq is not None, "no statistics output given")
+    if noise is not None:
+        _need(lse_pert is not None, "noise requires lse_pert")
+    lib = _lib.load()
+    st = lib.trn_attn_fwd_stats_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), None, _ptr(noise),
+                                    _ptr(lse_pert), _ptr(out_sum), _ptr(out_sumsq), _stream(q))
+    _lib.check("trn_attn_fwd_stats_f16", st)
+
+
 def prenorm_qkv(x: torch.Tensor, gamma: Optional[torch.Tensor], wq, wk, wv, q_out, k_out, v_out,
                 eps: float, norm: bool = True) -> None:
     """Q,K,V = RMSNorm(x; gamma, eps) @ W{q,k,v}  (norm=False: x @ W).
