@@ -229,3 +229,33 @@ def test_benchmark_cli_times_recognised_candidates_and_records_the_rest(tmp_path
     assert all(d["error"] is None and 0 < d["execution_time_ms"] < 10 for d in data if d["ir_id"] != 2)
     assert data[2]["error"].startswith("unsupported IR") and math.isinf(data[2]["execution_time_ms"])
     assert data[0]["ir_expression"].startswith("(seq (ploop")
+
+
+def test_printing_round_trips_on_random_trees():
+    """parse(str(tree)) == tree for randomly generated well-formed programs (hypothesis)."""
+    from hypothesis import given, settings, strategies as st
+    names = st.sampled_from(["X", "WQ", "K_cache", "O2", "C_sum", "noise", "T1"])
+    atoms = st.one_of(st.integers(-64, 4096), st.sampled_from(["m", "n", "p", "P+M", "N", "1.5"]))
+    idx = st.lists(st.one_of(st.just(ir.Node("fulltile")), st.builds(lambda v: ir.Node("tile", (v,)), st.sampled_from(["m", "n", "p"])),
+                             st.builds(lambda v: ir.Node("elem", (v,)), st.sampled_from(["h", "m"])),
+                             st.builds(lambda a, b: ir.Node("const_tile", (a, b)), atoms, atoms)), min_size=1, max_size=3)
+    index = st.builds(lambda xs: ir.Node("index", tuple(xs)), idx)
+    named = st.builds(lambda k, ns: ir.Node(k, tuple(ns)), st.sampled_from(["input", "output", "tensor"]), st.lists(names, min_size=1, max_size=3, unique=True))
+    load = st.builds(lambda t, i: ir.Node("load", (t, i)), named, index)
+    value = st.recursive(st.one_of(load, atoms), lambda kids: st.one_of(
+        st.builds(lambda op, a, b: ir.Node(op, (a, b)), st.sampled_from(["+", "-", "x", "/", "*"]), kids, kids),
+        st.builds(lambda op, a: ir.Node(op, (a,)), st.sampled_from(["exp", "sqr", "sqrt", "sigmoid"]), kids),
+        st.builds(lambda a, ax: ir.Node("rsum", (a, ax)), kids, st.integers(0, 2)),
+        st.builds(lambda a, ax: ir.Node("bcast", (a, ax)), kids, st.integers(0, 3))), max_leaves=8)
+    store = st.builds(lambda t, v, i: ir.Node("store", (t, v, i)), named, value, index)
+    stmt = st.recursive(st.one_of(store, st.just(ir.Node("dummy"))), lambda kids: st.one_of(
+        st.builds(lambda xs: ir.Node("seq", tuple(xs)), st.lists(kids, min_size=1, max_size=3)),
+        st.builds(lambda k, a, b, t, v, body: ir.Node(k, (a, b, t, v, body)), st.sampled_from(["ploop", "sloop"]), atoms, atoms,
+                  st.integers(1, 128), st.sampled_from(["m", "n", "p", "h"]), kids)), max_leaves=5)
+
+    @settings(max_examples=150, deadline=None)
+    @given(stmt)
+    def check(tree):
+        assert ir.parse(str(tree)) == tree
+        ir.recognise(tree)                       # never raises: a Match either way
+    check()
