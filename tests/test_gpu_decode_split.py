@@ -29,11 +29,11 @@ def workspace_for(q, k, v, o, scale, causal):
 
 SPLIT_CASES = [
     # B, Hq, Hkv, Sq, Skv, D, causal
-    (1, 32, 32, 16, 1040, 128, False),   # the reference's decode-append shape at Llama widths
-    (1, 32, 8, 16, 1040, 128, True),     # GQA, causal with a cached prefix
-    (1, 71, 1, 16, 2100, 64, False),     # Falcon: MQA, 71 heads of width 64
+    (1, 32, 32, 16, 2064, 128, False),   # twice the reference's decode-append cache at Llama widths
+    (1, 32, 8, 16, 1552, 128, True),     # GQA, causal with a cached prefix
+    (1, 71, 1, 16, 3100, 64, False),     # Falcon: MQA, 71 heads of width 64
     (2, 4, 2, 1, 4099, 128, True),       # one query, ragged keys, many shares
-    (1, 3, 1, 32, 1057, 128, True),      # 34 blocks in shares of 5: the last share is short
+    (1, 3, 1, 32, 1569, 128, True),      # 50 blocks in shares of 7: the last share is short
     (1, 8, 8, 7, 20000, 128, False),     # long cache
 ]
 
@@ -64,7 +64,7 @@ def test_split_keys_match_oracle_and_unsplit(B, Hq, Hkv, Sq, Skv, D, causal):
 
 def test_split_keys_with_noise_and_fused_q_norm():
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D = 1, 8, 2, 16, 1040, 128
+    B, Hq, Hkv, Sq, Skv, D = 1, 8, 2, 16, 1552, 128
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=3)
     noise = ref.gumbel_noise((B, Hq, Sq, Skv), 99)
     tau, scale = 1.5, D ** -0.5
@@ -89,7 +89,7 @@ def test_split_keys_with_noise_and_fused_q_norm():
 
 def test_workspace_rules():
     from triton_amd import ops, _lib
-    q, k, v = make(1, 8, 8, 16, 1040, 128)
+    q, k, v = make(1, 8, 8, 16, 1552, 128)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     o = torch.zeros_like(qd)
     scale = 128 ** -0.5
@@ -106,7 +106,7 @@ def test_workspace_rules():
         ops.attention(qd, kd, vd, o, scale, False, workspace=big[16:16 + n])
     assert e.value.status_name == "TRN_E_ALIGN"
     # shapes that do not split report 0 bytes: many heads, few keys, or more than 32 queries
-    for shape in ((1, 128, 128, 16, 1040, 128), (1, 8, 8, 16, 200, 128), (1, 8, 8, 33, 1040, 128)):
+    for shape in ((1, 128, 128, 16, 1552, 128), (1, 8, 8, 16, 1040, 128), (1, 8, 8, 33, 1552, 128)):
         qq, kk, vv = (t.cuda() for t in make(*shape))
         assert ops.attention_workspace_bytes(qq, kk, vv, torch.zeros_like(qq), scale, False) == 0
     # a workspace handed to a shape that does not use one is ignored
@@ -120,7 +120,7 @@ def test_workspace_rules():
 def test_split_keys_under_graph_replay():
     """Captured once, replayed with eager work between the replays: every replay gives the eager result."""
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 1040, 128
+    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 1552, 128
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=17)
     scale = D ** -0.5
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
@@ -148,10 +148,10 @@ def test_split_keys_under_graph_replay():
 
 
 def test_decode_modules_split_path_matches_reference_classes():
-    """The decode-append modules at a shape where the attention splits its keys (8 heads, 1040 keys); RoCo asks for
+    """The decode-append modules at a shape where the attention splits its keys (8 heads, 1552 keys); RoCo asks for
     the key statistics, which are a second sweep of the one workgroup per head, so it is not split."""
     from triton_amd import modules
-    M, N, D, P = 16, 1024, 128, 1024
+    M, N, D, P = 16, 1024, 128, 1536
     H = N // D
     g = torch.Generator().manual_seed(5)
     cpu = dict(X=ref.reference_recipe((M, N), g) * 30, WQ=ref.reference_recipe((N, N), g) * 30,

@@ -11,8 +11,11 @@
 // that the waits can be counted.
 #include "attn.h"
 
+// Memory order of the arrival increment.  Release/acquire at device scope makes the hand-over of the shares hold by
+// the memory model alone (the other threads' stores are ordered before it by the workgroup barrier); it costs one L2
+// write-back and one invalidate per WORKGROUP, about 1.5 us per launch.
 #ifndef TRN_ARRIVAL_ORDER
-#define TRN_ARRIVAL_ORDER __ATOMIC_RELAXED
+#define TRN_ARRIVAL_ORDER __ATOMIC_ACQ_REL
 #endif
 typedef unsigned long long ulong2_t __attribute__((ext_vector_type(2)));
 
@@ -273,7 +276,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         // {O as quads [D/4][32 queries][4], (m, l, m2, l2) [32]} floats.  The shares travel as device-scope atomic stores and loads, which
         // go to the memory all L2 slices agree on (a fence that makes ordinary stores visible writes back and
         // invalidates a whole L2, and with one per wave that took several times the kernel's own time); the arrival
-        // is a release/acquire increment by one thread, tied to the other threads by the workgroup barriers.
+        // is a release/acquire increment by ONE thread, tied to the other threads by the workgroup barriers.
         constexpr int PART = 32 * (D + 4);
         const int n_bh = a.B * a.Hq;
         unsigned* counters = reinterpret_cast<unsigned*>(a.ws);
@@ -416,13 +419,14 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 }
 
 // Keys are split over workgroups when one workgroup per head would leave most of the chip idle and a head has enough
-// key blocks to repay the merge: publishing, arriving and collecting cost about 4 us, which is what some 32 blocks of a
-// 128-wide head (twice as many of a 64-wide one) take a single workgroup.  Measured with 16 queries per head, 32 heads
-// of width 128: 1040 keys 14.8 -> 14.5 us, 4112 keys 43 -> 24 us, 16400 keys 154 -> 50 us; 8 heads, 16400 keys
-// 150 -> 26 us.  The caller provides the workspace for the partial results.
+// key blocks to repay the merge: publishing, arriving and collecting cost 4 - 5 us, which is what some 40 blocks of a
+// 128-wide head (twice as many of a 64-wide one) take a single workgroup; the threshold is 48.  Measured with 16
+// queries per head, 32 heads of width 128: 1040 keys 14.8 -> 16 us (hence not split), 2064 keys 24 -> 21 us, 4112
+// keys 43 -> 25 us, 16400 keys 154 -> 51 us; 8 heads, 16400 keys 150 -> 27 us.  The caller provides the workspace
+// for the partial results.
 static int decode_splits(int batch, int n_q_heads, int seq_kv, int head_dim) {
     const int n_bh = batch * n_q_heads, nblk = (seq_kv + 31) / 32;
-    if (n_bh >= 128 || (int64_t)nblk * head_dim < 32 * 128) return 1;
+    if (n_bh >= 128 || (int64_t)nblk * head_dim < 48 * 128) return 1;
     const int ns = max(1, min(min(16, 256 / n_bh), nblk / 4));
     const int bps = (nblk + ns - 1) / ns;                 // blocks per share, as the kernel computes it
     return (nblk + bps - 1) / bps;                        // no empty share: the last one starts inside the keys
