@@ -34,8 +34,10 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="default",
-                    help="default (vanilla headline + rmsnorm), all, or one of vanilla rmsnorm prenorm qknorm keyformer roco decode")
+    ap.add_argument("--workload", default="all",
+                    help="all (the headline, RMSNorm, the four other prefill workloads and the decode-append timings: the "
+                         "default), headline (vanilla attention + RMSNorm only), or one of vanilla rmsnorm prenorm qknorm "
+                         "keyformer roco decode")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="with --workload all: skip the decode-append timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
@@ -312,8 +314,8 @@ def main():
         del src, dst
     wl = a.workload
     extra = {}
-    van = bench_vanilla(a.steps, a.warmup) if wl in ("default", "all", "vanilla") else None
-    if wl in ("default", "all", "rmsnorm"):
+    van = bench_vanilla(a.steps, a.warmup) if wl in ("headline", "all", "vanilla") else None
+    if wl in ("headline", "all", "rmsnorm"):
         extra["rmsnorm"] = bench_rmsnorm(a.steps, a.warmup)
     for name in ("prenorm", "qknorm", "keyformer", "roco"):
         if wl in ("all", name):
