@@ -99,6 +99,39 @@ def test_validation_rejects_before_launch(lib):
     assert g(tokens=0) == 0
 
 
+def test_validation_of_the_workspace_statistics_and_linear_entry_points(lib):
+    """As above: every call fails validation before anything is launched."""
+    p = C.c_void_p(0x1000)
+    d = _desc()
+    ws = lambda w, n: lib.trn_attn_fwd_ws_f16(C.byref(d), p, p, p, p, None, None, None, None, w, n, None)
+    assert ws(C.c_void_p(0x1010), 4096) == -4                          # workspace not 256-byte aligned
+    assert lib.trn_attn_fwd_ws_f16(C.byref(d), None, p, p, p, None, None, None, None, p, 4096, None) == -1
+    assert lib.trn_attn_workspace_bytes(C.byref(_desc(head_dim=32))) == 0      # invalid shape: no workspace
+    assert lib.trn_attn_workspace_bytes(None) == 0
+    st = lambda dd, s1, s2: lib.trn_attn_fwd_stats_f16(C.byref(dd), p, p, p, p, None, None, None, None, s1, s2, None)
+    assert st(d, None, None) == -1                                     # no statistics output
+    assert st(_desc(q_norm=1), p, None) == -5                          # fused query norm is not offered with statistics
+    assert st(_desc(seq_q=64, seq_kv=64), p, None) == -1               # more than 32 queries: lse is the hand-over buffer
+    vps = lambda *xs: (C.c_void_p * len(xs))(*xs)
+    i64 = lambda *xs: (C.c_int64 * len(xs))(*xs)
+    lin = lambda tokens=4, hidden=64, ldx=64, k=1, n=(64,), ldw=(64,), ldo=(64,), w=None: lib.trn_linear_f16(
+        p, tokens, hidden, ldx, k, w if w is not None else vps(*([0x1000] * len(n))), i64(*n), i64(*ldw), vps(*([0x1000] * len(n))), i64(*ldo), None, None)
+    assert lin(k=0) == -2 and lin(k=4) == -2 and lin(hidden=60) == -2 and lin(n=(12,), ldw=(12,), ldo=(12,)) == -2
+    assert lin(ldx=32) == -3 and lin(ldw=(32,)) == -3 and lin(ldo=(68,)) == -4
+    assert lin(w=vps(None)) == -1 and lin(tokens=0) == 0
+    gate = lambda rows=4, cols=64, ld=64, kind=0, c1=p: lib.trn_gate_f16(c1, p, p, rows, cols, ld, ld, ld, kind, None)
+    assert gate(cols=12) == -2 and gate(kind=2) == -2 and gate(ld=32) == -3 and gate(ld=68) == -4
+    assert gate(c1=None) == -1 and gate(rows=0) == 0
+
+
+def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
+    from triton_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libtrinity_hip.so"))
+    with pytest.raises(ImportError, match="no fallback"):
+        _lib.load()
+
+
 def test_wrappers_raise_python_exceptions_on_cpu_tensors():
     from triton_amd import ops
     x = torch.zeros(4, 64, dtype=torch.float16)
