@@ -357,7 +357,7 @@ def main():
         "pct_of_fp16_mfma_peak": round(100 * van["tflops"] / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(van["kernel_tflops"], 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(van["kernel_tflops"] / peak, 4), "traffic": traffic,
-                     "kernel": "trn::attn_fwd_kernel<128, 8, false>", "kernel_ms": round(van["kernel_ms"], 5)},
+                     "kernel": "trn::attn_fwd16_kernel<128, 8>", "kernel_ms": round(van["kernel_ms"], 5)},
     }
     ceil = mfma_ceiling()
     line["roofline"]["mfma_only_kernel_tflops"] = {k: round(v, 1) for k, v in ceil.items()}

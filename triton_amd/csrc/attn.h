@@ -26,4 +26,7 @@ hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t
 // Bytes of workspace with which launch_attn_decode splits the keys of this problem over several workgroups (0: it would not).
 int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq_kv, int head_dim);
 
+// The forward pass without score perturbation on the 16x16x32 MFMA (attn_fwd16.hip); wide: 8 waves per workgroup.
+hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, bool wide, hipStream_t stream);
+
 }  // namespace trn

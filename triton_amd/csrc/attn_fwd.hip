@@ -1,4 +1,7 @@
-// Flash attention forward for gfx950: O = softmax(scale * Q K^T [+causal]) V, GQA/MQA, head_dim 64/128.
+// Flash attention forward for gfx950 on the 32x32x16 MFMA: O = softmax(scale * Q K^T [+causal]) V, GQA/MQA,
+// head_dim 64/128.  This file holds the entry points, and the kernel that runs when the scores are perturbed
+// (KeyFormer: one lane owns a whole query row here, which is what the noise stream wants); plain attention runs
+// on the 16x16x32 kernel of attn_fwd16.hip.
 //
 // Formulation.  Everything is computed TRANSPOSED so that a lane owns one query:
 //     S^T[key][query] = K[key][:] . Q[query][:]     (MFMA 32x32x16: A = K tile from LDS, B = Q^T in registers)
@@ -506,7 +509,10 @@ static int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* 
 #else
     const bool wide = TRN_FORCE_NW == 8;
 #endif
-#define TRN_LAUNCH(D_, NW_) (noise ? launch_fwd<D_, NW_, true>(a, s) : launch_fwd<D_, NW_, false>(a, s))
+    // Without score perturbation: the 16x16x32 kernel; with head_dim 64 always its 4-wave form (measured: the 8-wave
+    // form loses 10-20 % there, at every size).
+    if (!noise) return launch_attn_fwd16(a, d->head_dim, wide && d->head_dim == 128, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+#define TRN_LAUNCH(D_, NW_) launch_fwd<D_, NW_, true>(a, s)
     if (d->head_dim == 128) e = wide ? TRN_LAUNCH(128, 8) : TRN_LAUNCH(128, 4);
     else e = wide ? TRN_LAUNCH(64, 8) : TRN_LAUNCH(64, 4);
 #undef TRN_LAUNCH

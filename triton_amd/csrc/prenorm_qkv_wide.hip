@@ -30,7 +30,9 @@ namespace trn {
 // x four consecutive chunks of one phase of the transposing read touch every bank once.
 __device__ __forceinline__ int gswz(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
 
-template <int NB>
+// G: gamma is multiplied into the X operand (norm on and a gamma given); without it the multiply, the gamma
+// loads and their ring leave the loop.
+template <int NB, bool G>
 __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
     // One array per stage and operand: the compiler orders LDS reads after outstanding global->LDS loads that may
@@ -104,8 +106,7 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
 #define TRN_FETCH(kt_, xd_, wd_) _Pragma("unroll") for (int fi_ = 0; fi_ < 4; ++fi_) TRN_FETCH_ONE(kt_, xd_, wd_, fi_)
 
     // ---- gamma: the X^T operand of contraction step ks holds columns kt*32 + ks*16 + 8h .. +7 of its token.
-    // Without a gamma the multiplier is 1.0, an exact no-op, so that the loop has one form.
-    const bool use_g = a.gamma != nullptr && a.norm;
+    constexpr bool use_g = G;
     const bool stats = a.norm && wn == 0;
     const __amdgpu_buffer_rsrc_t grs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(use_g ? a.gamma : a.x), 0, use_g ? a.K * 2 : 0, 0x00020000);
@@ -183,7 +184,7 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
             }
             __builtin_amdgcn_sched_barrier(0);
             acc[2][mb] = mfma32(wa[2], xv, acc[2][mb]);
-            const half8_t xv_next = raw * (mb < 3 ? g : gn);
+            const half8_t xv_next = G ? raw * (mb < 3 ? g : gn) : raw;
             if constexpr (NB == 4) {
                 if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
                 if (mb == 1) wn_[3] = read_w(Wr, ks_r, 3);
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
             ss[0] = __builtin_amdgcn_fdot2(p, p, ss[0], false);
         }
     }
-    xv = xv * g0[0];
+    if (G) xv = xv * g0[0];
 
     // k-tile kt reads stage kt%4: the operands of its first step during the second step of k-tile kt-1, those of
     // its second step during its first.  From the barrier between the two steps on, the stage is free and is
@@ -340,8 +341,10 @@ int launch_prenorm_qkv_wide(GemmArgs a, hipStream_t stream) {
     a.panels_per_xcd = (a.n_panels + 7) / 8;
     const int64_t grid = (int64_t)8 * a.panels_per_xcd * a.n_mtiles;
     if (grid > 0x7fffffffLL) return TRN_E_SHAPE;
-    if (nb == 3) hipLaunchKernelGGL(prenorm_qkv_wide_kernel<3>, dim3((unsigned)grid), dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(prenorm_qkv_wide_kernel<4>, dim3((unsigned)grid), dim3(256), 0, stream, a);
+    const bool g = a.gamma != nullptr && a.norm;
+    auto* kernel = nb == 3 ? (g ? prenorm_qkv_wide_kernel<3, true> : prenorm_qkv_wide_kernel<3, false>)
+                           : (g ? prenorm_qkv_wide_kernel<4, true> : prenorm_qkv_wide_kernel<4, false>);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(256), 0, stream, a);
     return hipGetLastError() == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 }
 
