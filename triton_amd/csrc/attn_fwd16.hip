@@ -301,9 +301,22 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         step(needs_mask(kv0 + 32), std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
         step(needs_mask(kv0 + 64), std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
     };
-    for (int jt = 0; jt < ntiles; jt += 2) {
+    // Under a causal mask the waves of a workgroup see different numbers of tiles: a wave computes the tiles that
+    // hold a key visible to one of its queries, and for the rest only keeps up the staging it shares with the
+    // others (its part of every refill, and the barrier), leaving its SIMD to the wave that still computes.
+    int nlive = ntiles;
+    if (a.causal) nlive = min(ntiles, (min(wq0 + 31, a.Sq - 1) + off) / BN + 1);
+    for (int jt = 0; jt < nlive; jt += 2) {
         tile(jt, Ks0, Ks1, Vs0, Vs1);
-        if (jt + 1 < ntiles) tile(jt + 1, Ks1, Ks0, Vs1, Vs0);
+        if (jt + 1 < nlive) tile(jt + 1, Ks1, Ks0, Vs1, Vs0);
+    }
+    for (int jt = nlive; jt < ntiles; ++jt) {
+        half_t* Kc = (jt & 1) ? Ks1 : Ks0;
+        half_t* Vn = (jt & 1) ? Vs0 : Vs1;
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
+        if (jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
     }
 #undef TRN_FETCH_K
 #undef TRN_FETCH_V
