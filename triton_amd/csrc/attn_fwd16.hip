@@ -135,7 +135,10 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
 #pragma unroll
     for (int i = 0; i < NOP; ++i) oacc[i][0] = oacc[i][1] = zero;
     float m[2] = {-INFINITY, -INFINITY};    // reference max (log2 domain), equal in the four lanes of a query
-    float l[2] = {0.f, 0.f};                // this lane's partial row sums
+    // Row sums come out of the matrix pipe as well: one more MFMA per query block whose A operand is all ones leaves
+    // the sum of the block's (fp16-rounded) probabilities of each query in every row of a 16 x 16 accumulator.  Two
+    // MFMAs per 32-key block instead of eight dot-product instructions, each of which costs two VALU issue slots.
+    float4_t lacc[2] = {zero, zero};
 
     int ntiles = (a.Skv + BN - 1) / BN;
     if (a.causal) ntiles = min(ntiles, (min(q0 + BM - 1, a.Sq - 1) + off) / BN + 1);
@@ -189,7 +192,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         for (int qb = 0; qb < 2; ++qb) {
             const float mnew = fmaxf(m[qb], quad_max(smax[qb]));
             const float alpha = fast_exp2(m[qb] - mnew);
-            l[qb] *= alpha;
+            lacc[qb] = lacc[qb] * alpha;
 #pragma unroll
             for (int i = 0; i < NOP; ++i)
                 oacc[i][qb] = oacc[i][qb] * alpha;      // (as one vector operation: written per element, the path that
@@ -198,6 +201,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         }
     };
 
+    const half_t one = (half_t)1.f;
+    const half8_t ones8 = {one, one, one, one, one, one, one, one};
     constexpr int NQ = 2;   // operand look-ahead, in operands (= 2 NQ MFMA slots; 4 measured no better)
     static_assert(NOP % NQ == 0, "the operand window must divide the operands of a phase");
     half8_t ka[NQ];    // K operands of the next block's S^T, a rolling window ahead of use
@@ -215,7 +220,6 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     auto step = [&](bool masked_next, auto sync_tag, Scores16& sc, Scores16& sn, const half_t* Vblk, const half_t* K1,
                     const half_t* K2, int key0_next, auto&& handover) __attribute__((always_inline)) {
         constexpr bool SYNC = decltype(sync_tag)::value;
-        const half2_t ones = {(half_t)1.f, (half_t)1.f};
         half8_t pB[2];
         auto load_v = [&](int db, int reg) __attribute__((always_inline)) {
             const half4_t lo = lds_read_tr16(Vblk + voff[db]);              // keys 4 g4 .. +3, dim 16 db + n
@@ -227,7 +231,6 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             const float p0 = fast_exp2(__builtin_fmaf(sc.s[kb][qb][i0], a.c1, -m[qb]));
             const float p1 = fast_exp2(__builtin_fmaf(sc.s[kb][qb][i0 + 1], a.c1, -m[qb]));
             const half2_t pp = {(half_t)p0, (half_t)p1};
-            l[qb] = __builtin_amdgcn_fdot2(pp, ones, l[qb], false);      // the sum runs over the fp16-rounded P
             pB[qb][4 * kb + i0] = pp[0]; pB[qb][4 * kb + i0 + 1] = pp[1];
         };
         // ---- phase A ----
@@ -260,6 +263,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             if (i == NS / 2) due = reduce_block(masked_next, sn, key0_next, smax);
             __builtin_amdgcn_sched_barrier(0);
         }
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) lacc[qb] = mfma16(ones8, pB[qb], lacc[qb]);
         if (due) rescale(smax);
     };
 
@@ -324,8 +329,9 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     // ---- epilogue: normalise; transpose this wave's 32 x D tile through LDS so that the stores are whole
     // 16-byte-per-lane row segments; LSEs ----
     float inv[2];
+    float l[2];
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) { l[qb] = quad_sum(l[qb]); inv[qb] = 1.0f / l[qb]; }
+    for (int qb = 0; qb < 2; ++qb) { l[qb] = lacc[qb][0]; inv[qb] = 1.0f / l[qb]; }
     __syncthreads();                                   // every wave is done with the K/V stages
     {
         // two passes of D/2 columns each, so that NW waves' staging regions fit in the four stage arrays
