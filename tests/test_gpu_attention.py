@@ -47,6 +47,9 @@ CASES = [
     (1, 4, 2, 32, 32, 128, True),
     (3, 4, 4, 32, 5000, 128, False),
     (1, 4, 2, 33, 1040, 128, True),      # one query more: back to the prefill kernel
+    (1, 64, 8, 1990, 2100, 128, True),   # 8-wave workgroups under a causal mask with a cached prefix and ragged ends:
+                                         # the waves of a workgroup stop at different tiles
+    (1, 16, 16, 520, 520, 64, True),     # head_dim 64 stays on 4-wave workgroups; a last workgroup of 8 queries
 ]
 
 
@@ -116,6 +119,19 @@ def test_qnorm_fused():
     ops.attention(q.cuda(), kn, v.cuda(), od, D ** -0.5, True, q_norm=True, gamma_q=gq.cuda(), q_eps=1e-5)
     torch.cuda.synchronize()
     close(od, ref.qknorm_attention(q, k, v, gq, gk, 1e-5, D ** -0.5, True))
+
+
+def test_qnorm_fused_head_dim_128_no_gamma():
+    """The query norm of the 16x16x32 kernel sums a row over four lanes; without a weight and with eps = 0 it is the
+    reference's QKNorm statement (q * rsqrt(mean(q^2)))."""
+    from triton_amd import ops
+    B, Hq, Hkv, S, D = 2, 4, 2, 300, 128
+    q, k, v = make(B, Hq, Hkv, S, S, D, seed=21)
+    od = torch.zeros_like(q).cuda()
+    ops.attention(q.cuda(), k.cuda(), v.cuda(), od, D ** -0.5, True, q_norm=True, gamma_q=None, q_eps=0.0)
+    torch.cuda.synchronize()
+    qn = ref.rmsnorm(q, torch.ones(D, dtype=torch.float16), 0.0)
+    close(od, ref.attention(qn, k, v, D ** -0.5, True))
 
 
 def test_noise_row_normaliser():
