@@ -68,6 +68,39 @@ def test_attention_parity(B, Hq, Hkv, Sq, Skv, D, causal):
     close(lse, want_lse, atol=1e-3, rtol=1e-3)
 
 
+def _random_shapes(n, seed):
+    import random
+    rnd = random.Random(seed)
+    out = []
+    for _ in range(n):
+        D = rnd.choice((64, 128))
+        Hkv = rnd.choice((1, 2, 3))
+        Hq = Hkv * rnd.choice((1, 2, 4))
+        B = rnd.choice((1, 2))
+        causal = rnd.random() < 0.6
+        Sq = rnd.choice((33, 40, 64, 97, 128, 129, 200, 255, 256, 257, 300, 384, 511, 513, 640))
+        Skv = Sq + rnd.choice((0, 0, 1, 31, 32, 33, 64, 100, 257)) if causal else rnd.choice((1, 17, 32, 63, 64, 65, 200, 333, 512, 700))
+        out.append((B, Hq, Hkv, Sq, Skv, D, causal, rnd.random() < 0.3))
+    return out
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,qnorm", _random_shapes(48, 20260101))
+def test_attention_parity_seeded_random_shapes(B, Hq, Hkv, Sq, Skv, D, causal, qnorm):
+    """A seeded sweep over ragged query / key counts on both sides of the 32-, 64- and 256-row tile edges, GQA ratios,
+    cached prefixes of every alignment, both head widths, with and without the fused query norm."""
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=Sq * 1000 + Skv)
+    scale = D ** -0.5
+    od = torch.zeros_like(q).cuda()
+    lse = torch.zeros(B, Hq, Sq, dtype=torch.float32, device="cuda")
+    ops.attention(q.cuda(), k.cuda(), v.cuda(), od, scale, causal, lse=lse, q_norm=qnorm, gamma_q=None, q_eps=0.0)
+    torch.cuda.synchronize()
+    qq = ref.rmsnorm(q, torch.ones(D, dtype=torch.float16), 0.0) if qnorm else q
+    want, want_lse = ref.attention(qq, k, v, scale, causal, return_lse=True)
+    close(od, want)
+    close(lse, want_lse, atol=1e-3, rtol=1e-3)
+
+
 def test_attention_reference_recipe_unscaled():
     """The reference's own input recipe and semantics: scale 1, no mask (ref_rms.py:77-78)."""
     from triton_amd import ops
