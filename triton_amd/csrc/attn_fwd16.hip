@@ -11,9 +11,9 @@
 //     S^T(kb, qb)[key][query] = K[16 kb + key][:] . Q[16 qb + query][:]   A = K rows from LDS (one 16-byte read:
 //                               row n, contraction columns 32 ks + 8 g ..+7), B = Q^T in registers
 //   the lane receives keys 16 kb + 4 g + 0..3 of its two queries: 8 keys per query, the other 24 sit in the
-//   lanes n + 16, n + 32, n + 48.  Row sums stay per lane until the end; the running max is kept equal in the four
-//   lanes of a query, and whether it must rise is decided from the lane's own 8 keys (any lane of the wave
-//   over the threshold raises it for all), so the common path has no cross-lane traffic at all.
+//   lanes n + 16, n + 32, n + 48.  The running max is kept equal in the four lanes of a query, and whether it must
+//   rise is decided from the lane's own 8 keys (any lane of the wave over the threshold raises it for all), so the
+//   common path has no cross-lane traffic at all.  Row sums come from the matrix pipe (an all-ones A operand).
 //     O^T(db, qb)[d][query] += V^T[16 db + d][slot] * P^T[slot][query]   one MFMA per 32-key block (K = 32)
 //   contraction slot 8 g + j of a lane is key 4 g + j (j < 4) or 16 + 4 g + (j - 4): exactly the keys whose
 //   scores the lane holds, so P goes from the S^T accumulators to the B operand without leaving the lane, and the
