@@ -38,7 +38,8 @@ typedef enum trn_status {
     TRN_E_ALIGN       = -4,  /* pointer or pitch not 16-byte aligned                      */
     TRN_E_UNSUPPORTED = -5,  /* e.g. head_dim not in {64,128}                             */
     TRN_E_LAUNCH      = -6,  /* the HIP runtime refused the launch                        */
-    TRN_E_ARCH        = -7   /* current device is not gfx950                              */
+    TRN_E_ARCH        = -7,  /* current device is not gfx950                              */
+    TRN_E_SCRATCH     = -8   /* the problem needs more scratch memory than the library's static buffer holds */
 } trn_status;
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -47,8 +48,9 @@ int trn_version(void);
 /* Static string naming a trn_status value ("TRN_E_SHAPE"...). */
 const char* trn_status_name(int status);
 
-/* 0 if the current HIP device is a gfx950, TRN_E_ARCH otherwise.  Not capture-safe
- * (queries device properties); call once at load time. */
+/* 0 if the current HIP device is a gfx950, TRN_E_ARCH otherwise.  Also looks up, for this device, the
+ * address of the static scratch array behind trn_attn_fwd_noalloc_f16.  Not capture-safe (queries
+ * device properties); call once per device at load time. */
 int trn_check_device(void);
 
 /*
@@ -122,6 +124,23 @@ int trn_attn_fwd_ws_f16(const trn_attn_desc* desc, const void* q, const void* k,
                         void* o, float* lse, const void* gamma_q,
                         const float* noise, float* lse_pert,
                         void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
+ * trn_attn_fwd_ws_f16 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): it has no counterpart in the reference.  The workspace is a static device
+ * array inside the library, TRN_ATTN_NOALLOC_SCRATCH_BYTES per GPU, held from load until the process ends; the call
+ * itself allocates and frees nothing.  A problem whose workspace (trn_attn_workspace_bytes) would be larger is
+ * rejected with TRN_E_SCRATCH; one that needs none runs as trn_attn_fwd_f16.  The arrival counters are cleared by a
+ * small kernel on `stream` before the attention kernel, so a call does not depend on what the previous one left.
+ * All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race; serialise
+ * them, or give overlapping callers their own workspace through trn_attn_fwd_ws_f16.  Call trn_check_device once
+ * per device first if the call is to be captured into a graph (the first call on a device otherwise looks up the
+ * array's address itself, which is not a stream operation).
+ */
+#define TRN_ATTN_NOALLOC_SCRATCH_BYTES (8u << 20)
+int trn_attn_fwd_noalloc_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                             void* o, float* lse, const void* gamma_q,
+                             const float* noise, float* lse_pert, void* stream);
 
 /*
  * Per-key column statistics of the attention probabilities, given the row normalisers from

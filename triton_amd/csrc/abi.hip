@@ -1,5 +1,5 @@
 // Library-level entry points: version, status names, device check.
-#include "common.h"
+#include "attn.h"
 #include <string.h>
 
 extern "C" int trn_version(void) { return 100; }  // 0.1.0
@@ -14,6 +14,7 @@ extern "C" const char* trn_status_name(int status) {
         case TRN_E_UNSUPPORTED: return "TRN_E_UNSUPPORTED";
         case TRN_E_LAUNCH: return "TRN_E_LAUNCH";
         case TRN_E_ARCH: return "TRN_E_ARCH";
+        case TRN_E_SCRATCH: return "TRN_E_SCRATCH";
         default: return "TRN_E_UNKNOWN";
     }
 }
@@ -23,7 +24,9 @@ extern "C" int trn_check_device(void) {
     if (hipGetDevice(&dev) != hipSuccess) return TRN_E_ARCH;
     hipDeviceProp_t prop;
     if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return TRN_E_ARCH;
-    return strncmp(prop.gcnArchName, "gfx950", 6) == 0 ? TRN_OK : TRN_E_ARCH;
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return TRN_E_ARCH;
+    // set-up that must not happen under graph capture: the address of the static scratch array on this device
+    return trn::attn_static_scratch() ? TRN_OK : TRN_E_LAUNCH;
 }
 
 // Plain streaming copy, 16 bytes per lane, non-temporal both ways: the yardstick that HBM counters and

@@ -21,10 +21,19 @@ struct AttnArgs {
     float* col_sum; float* col_sumsq;
 };
 
+// Checks, argument block and kernel choice behind every attention entry point of the C ABI.
+int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
+                 const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
+                 int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream);
+
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream);
 // Bytes of workspace with which launch_attn_decode splits the keys of this problem over several workgroups (0: it would not).
 int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq_kv, int head_dim);
+
+// Device address, on the current device, of the library's static scratch array (TRN_ATTN_NOALLOC_SCRATCH_BYTES bytes)
+// behind trn_attn_fwd_noalloc_f16; looked up once per device.  nullptr if the runtime refuses.
+void* attn_static_scratch();
 
 // The forward pass without score perturbation on the 16x16x32 MFMA (attn_fwd16.hip); wide: 8 waves per workgroup.
 hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, bool wide, hipStream_t stream);

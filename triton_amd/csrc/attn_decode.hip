@@ -10,6 +10,7 @@
 // loop has no barrier; every load is issued unconditionally (blocks past the end read zeros, which are masked) so
 // that the waits can be counted.
 #include "attn.h"
+#include <mutex>
 
 // Memory order of the arrival increment.  Release/acquire at device scope makes the hand-over of the shares hold by
 // the memory model alone (the other threads' stores are ordered before it by the workgroup barrier); it costs one L2
@@ -461,3 +462,60 @@ hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t
 }
 
 }  // namespace trn
+
+// ---- the entry point that allocates nothing ------------------------------------------------------------------------
+// The split-key path needs device memory beyond its inputs and outputs (arrival counters and the shares' partial
+// results).  For callers that cannot allocate, that memory is a file-scope device array: every GPU the library runs
+// on holds its own copy of it, at its own address, until the process ends.  On the host the array's NAME is only a
+// handle for hipGetSymbolAddress; the address that kernels, fills and copies take is the one that call returns for
+// the device that is current, looked up once per device and kept.
+static __device__ __align__(256) unsigned char scratch[TRN_ATTN_NOALLOC_SCRATCH_BYTES];
+
+namespace trn {
+
+constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxDevices];      // device address of `scratch` on each device, null until looked up
+
+// Device address of the scratch array on the current device (looked up on first use; nothing is allocated: the
+// array is part of the code object).  Returns nullptr if the runtime refuses.
+void* attn_static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = p;
+    }
+    return g_scratch_ptr[dev];
+}
+
+// Zeroes n dwords (a kernel rather than a memset node, so that the call can be recorded into a graph).
+__global__ __launch_bounds__(256) void fill_zero_kernel(unsigned* p, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+}  // namespace trn
+
+extern "C" int trn_attn_fwd_noalloc_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                        float* lse, const void* gamma_q, const float* noise, float* lse_pert,
+                                        void* stream) {
+    using namespace trn;
+    if (!d) return TRN_E_NULL;
+    const int64_t need = trn_attn_workspace_bytes(d);
+    if (need == 0)      // a shape whose kernels use no scratch memory (or an invalid one: reported by the checks below)
+        return attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, nullptr, nullptr, stream);
+    if (need > (int64_t)TRN_ATTN_NOALLOC_SCRATCH_BYTES) return TRN_E_SCRATCH;
+    void* ws = attn_static_scratch();
+    if (!ws) return TRN_E_LAUNCH;
+    // The array keeps whatever the last call on this device left.  The shares are rewritten by every launch before
+    // they are read; the arrival counters must start at zero, so they are cleared here (the kernel also leaves them
+    // at zero, but a launch that failed half way would not have).
+    const int n_counters = (int)(((int64_t)d->batch * d->n_q_heads + 63) / 64) * 64;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((n_counters + 255) / 256), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<unsigned*>(ws), n_counters);
+    if (hipGetLastError() != hipSuccess) return TRN_E_LAUNCH;
+    return attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, ws, TRN_ATTN_NOALLOC_SCRATCH_BYTES, nullptr, nullptr, stream);
+}

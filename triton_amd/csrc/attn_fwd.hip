@@ -424,12 +424,6 @@ extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const voi
     return trn_attn_fwd_ws_f16(d, q, k, v, o, lse, gamma_q, noise, lse_pert, nullptr, 0, stream);
 }
 
-namespace trn {
-static int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
-                        const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
-                        int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream);
-}
-
 extern "C" int trn_attn_fwd_ws_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
                                    float* lse, const void* gamma_q, const float* noise, float* lse_pert,
                                    void* workspace, int64_t workspace_bytes, void* stream) {
@@ -456,7 +450,7 @@ extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, con
     return trn_attn_colstats_f16(d, q, k, rows, noise, out_sum, out_sumsq, stream);
 }
 
-static int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
+int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
                              const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
                              int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream) {
     if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;

@@ -112,7 +112,8 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
     """o = softmax(scale * q k^T [+causal]) v.  q,o [B,Hq,Sq,D]; k,v [B,Hkv,Skv,D] (strided views allowed).
     Optional outputs: lse [B,Hq,Sq] fp32; with noise [B,Hq,Sq,Skv] fp32 also lse_pert.
     workspace: optional zero-initialised uint8 tensor of attention_workspace_bytes(...) bytes (decode shapes with
-    few heads then split their keys over several workgroups)."""
+    few heads then split their keys over several workgroups); the string "static" takes the library's own static
+    device array instead (nothing is allocated; one such call at a time per GPU)."""
     d = _attn_desc(q, k, v, o, scale, causal, q_norm, q_eps, noise, tau)
     B, Hq, Sq, _ = q.shape
     _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq))
@@ -121,6 +122,12 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
         _need(gamma_q.shape == (q.shape[3],), "gamma_q: expected (head_dim,)")
     _need(noise is None or lse_pert is not None, "noise given without lse_pert")
     lib = _lib.load()
+    if isinstance(workspace, str):
+        _need(workspace == "static", 'workspace: a uint8 GPU tensor, None, or "static"')
+        st = lib.trn_attn_fwd_noalloc_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
+                                          _ptr(noise), _ptr(lse_pert), _stream(q))
+        _lib.check("trn_attn_fwd_noalloc_f16", st)
+        return
     if workspace is not None:
         _need(workspace.is_cuda and workspace.is_contiguous() and workspace.dtype == torch.uint8, "workspace: expected a contiguous uint8 GPU tensor")
         st = lib.trn_attn_fwd_ws_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
