@@ -18,6 +18,10 @@
 //   contraction slot 8 g + j of a lane is key 4 g + j (j < 4) or 16 + 4 g + (j - 4): exactly the keys whose
 //   scores the lane holds, so P goes from the S^T accumulators to the B operand without leaving the lane, and the
 //   A operand takes its two transposing reads from rows 4 g .. and 16 + 4 g .. of the V stage.
+// The exponent comes out of the matrix pipe ready-made: Q is multiplied by scale * log2(e) once in the prologue, and
+// every score chain starts from the accumulator {-m} instead of zero, so S^T arrives as s - m and the softmax costs
+// one v_exp_f32 per score and nothing else (the multiply-subtract it replaces was a quarter of the loop's vector
+// instructions).  When the lazy maximum rises, the scores already in flight are shifted along with it.
 // Staging (global -> LDS loads, XOR swizzle, two stages each for K and V, one barrier per 64-key tile), the grid
 // and the lazy running maximum are those of attn_fwd.hip.
 #include "attn.h"
@@ -94,7 +98,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * g4;
 #pragma unroll
         for (int ks = 0; ks < NKS; ++ks) qB[qb][ks] = *reinterpret_cast<const half8_t*>(qp + ks * 32);
-        if (a.q_norm) {   // fused per-head RMSNorm of the query row (the rest of the row is in the lanes n + 16, + 32, + 48)
+        const bool q_norm = a.q_norm != 0;
+        if (q_norm) {   // fused per-head RMSNorm of the query row (the rest of the row is in the lanes n + 16, + 32, + 48)
             float ss = 0.f;
 #pragma unroll
             for (int ks = 0; ks < NKS; ++ks)
@@ -114,6 +119,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
                 }
             }
         }
+        // the softmax scale and log2(e) go into Q once, so that the scores leave the matrix pipe ready for exp2
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qB[qb][ks][e] = (half_t)((float)qB[qb][ks][e] * a.c1);
     }
 
     // ---- LDS read offsets (halfs).  K operand (ks, kb): row 16 kb + n of a 32-key block, logical chunk 4 ks + g4
@@ -135,6 +145,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
 #pragma unroll
     for (int i = 0; i < NOP; ++i) oacc[i][0] = oacc[i][1] = zero;
     float m[2] = {-INFINITY, -INFINITY};    // reference max (log2 domain), equal in the four lanes of a query
+    float4_t negm[2];                       // {-m} x 4: the initial accumulator of every score chain, so that the
+                                            // scores arrive as s - m and the exponential needs no subtraction
     // Row sums come out of the matrix pipe as well: one more MFMA per query block whose A operand is all ones leaves
     // the sum of the block's (fp16-rounded) probabilities of each query in every row of a 16 x 16 accumulator.  Two
     // MFMAs per 32-key block instead of eight dot-product instructions, each of which costs two VALU issue slots.
@@ -182,16 +194,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             const float4_t& u = sx.s[0][qb];
             const float4_t& w = sx.s[1][qb];
             smax[qb] = fmaxf(max3(u[0], u[1], u[2]), max3(u[3], w[0], w[1]));
-            smax[qb] = max3(smax[qb], w[2], w[3]) * a.c1;
-            over = over || smax[qb] > m[qb] + 8.0f;
+            smax[qb] = max3(smax[qb], w[2], w[3]);
+            over = over || smax[qb] > 8.0f;
         }
         return __builtin_amdgcn_ballot_w64(over) != 0;
     };
-    auto rescale = [&](const float (&smax)[2]) __attribute__((always_inline)) {
+    // smax is relative to m, and so are the scores sx already in flight: they move with it
+    auto rescale = [&](const float (&smax)[2], Scores16& sx) __attribute__((always_inline)) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
-            const float mnew = fmaxf(m[qb], quad_max(smax[qb]));
-            const float alpha = fast_exp2(m[qb] - mnew);
+            const float up = fmaxf(0.f, quad_max(smax[qb]));
+            const float mnew = m[qb] + up;
+            const float alpha = fast_exp2(-up);
+            sx.s[0][qb] = sx.s[0][qb] - up;
+            sx.s[1][qb] = sx.s[1][qb] - up;
+            negm[qb] = float4_t{-mnew, -mnew, -mnew, -mnew};
             lacc[qb] = lacc[qb] * alpha;
 #pragma unroll
             for (int i = 0; i < NOP; ++i)
@@ -228,9 +245,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         };
         auto exp_pair = [&](int p) __attribute__((always_inline)) {        // scores 2 (p%2), +1 of key half (p/2)%2, query block p/4
             const int qb = p >> 2, kb = (p >> 1) & 1, i0 = 2 * (p & 1);
-            const float p0 = fast_exp2(__builtin_fmaf(sc.s[kb][qb][i0], a.c1, -m[qb]));
-            const float p1 = fast_exp2(__builtin_fmaf(sc.s[kb][qb][i0 + 1], a.c1, -m[qb]));
-            const half2_t pp = {(half_t)p0, (half_t)p1};
+            const float p0 = fast_exp2(sc.s[kb][qb][i0]);
+            const float p1 = fast_exp2(sc.s[kb][qb][i0 + 1]);
+            uint32_t u = pack_half2(p0, p1);
+            asm volatile("" : "+v"(u));     // keeps the pair's work in this slot (it is otherwise sunk past the hand-over)
+            const half2_t pp = __builtin_bit_cast(half2_t, u);
             pB[qb][4 * kb + i0] = pp[0]; pB[qb][4 * kb + i0 + 1] = pp[1];
         };
         // ---- phase A ----
@@ -240,7 +259,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             if constexpr (SYNC) {
                 if (i == NS - 2 * NQ) handover();
             }
-            sn.s[kb][qb] = mfma16(ka[op % NQ], qB[qb][ks], ks == 0 ? zero : sn.s[kb][qb]);
+            sn.s[kb][qb] = mfma16(ka[op % NQ], qB[qb][ks], ks == 0 ? negm[qb] : sn.s[kb][qb]);
             if (i & 1) {
                 if (op + NQ < NOP) load_k(K1, op + NQ, op % NQ);
                 else load_v(op + NQ - NOP, op % NQ);
@@ -265,7 +284,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         }
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) lacc[qb] = mfma16(ones8, pB[qb], lacc[qb]);
-        if (due) rescale(smax);
+        if (due) rescale(smax, sn);
     };
 
     // ---- prologue: K stages 0 and 1 and V stage 0; scores of block 0; first K operands of block 1 ----
@@ -287,8 +306,16 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             }
 #pragma unroll
         for (int i = 0; i < NQ; ++i) load_k(Ks0 + 32 * D, i, i);
+        // block 0 sets the reference outright (every query sees key 0, so it is finite from here on)
         float smax[2];
-        if (reduce_block(true, sA, 0, smax)) rescale(smax);
+        reduce_block(true, sA, 0, smax);
+#pragma unroll
+        for (int qb = 0; qb < 2; ++qb) {
+            m[qb] = quad_max(smax[qb]);
+            negm[qb] = float4_t{-m[qb], -m[qb], -m[qb], -m[qb]};
+            sA.s[0][qb] = sA.s[0][qb] - m[qb];
+            sA.s[1][qb] = sA.s[1][qb] - m[qb];
+        }
     }
 
     // One 64-key tile jt.  Kc = its own K stage (block 1 still has operands to give), Kn = the next tile's
