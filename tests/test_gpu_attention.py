@@ -50,6 +50,12 @@ CASES = [
     (1, 64, 8, 1990, 2100, 128, True),   # 8-wave workgroups under a causal mask with a cached prefix and ragged ends:
                                          # the waves of a workgroup stop at different tiles
     (1, 16, 16, 520, 520, 64, True),     # head_dim 64 stays on 4-wave workgroups; a last workgroup of 8 queries
+    # causal grids of a single round run "paired" (a workgroup's two wave groups own 128-query tiles from opposite
+    # ends of the sequence): an odd tile count (the middle tile is alone), ragged ends, a cached prefix, both widths
+    (1, 96, 8, 600, 600, 128, True),
+    (1, 96, 8, 600, 700, 128, True),
+    (2, 64, 64, 500, 500, 64, True),
+    (1, 32, 8, 2048, 2048, 128, True),   # the attention of the PreNorm block (BASELINE config 3)
 ]
 
 

@@ -13,6 +13,7 @@ struct AttnArgs {
     float c2, c3;  // scale*log2(e)/tau, log2(e)/tau     : perturbed scores  z2 = s*c2 + g*c3
     float q_eps;
     int causal, q_norm;
+    int paired;    // attn_fwd16 only: a workgroup's two wave groups own query tiles from opposite ends (set by its launcher)
     // decode kernel only: keys split over n_split workgroups per head, partial results and arrival counters in ws
     int n_split;
     float* ws;
@@ -35,7 +36,13 @@ int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq
 // behind trn_attn_fwd_noalloc_f16; looked up once per device.  nullptr if the runtime refuses.
 void* attn_static_scratch();
 
-// The forward pass without score perturbation on the 16x16x32 MFMA (attn_fwd16.hip); wide: 8 waves per workgroup.
-hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, bool wide, hipStream_t stream);
+// The forward pass without score perturbation on the 16x16x32 MFMA (attn_fwd16.hip).  Narrow: 4 waves x 32 queries
+// per workgroup; Wide: 8 waves x 32 consecutive queries; Paired: 8 waves, two 128-query tiles from opposite ends of
+// the sequence (causal problems whose grid is a single round).
+enum class Attn16Shape { Narrow, Wide, Paired };
+Attn16Shape attn_fwd16_shape(int batch, int n_q_heads, int seq_q, int head_dim, bool causal);
+hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, Attn16Shape shape, hipStream_t stream);
+// Name of the kernel instantiation that launch_attn_fwd16 runs for this shape, as a profiler prints it.
+const char* attn_fwd16_kernel_name(int head_dim, Attn16Shape shape);
 
 }  // namespace trn

@@ -483,7 +483,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
-    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq;
+    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.paired = 0;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
     if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)
@@ -493,19 +493,14 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     // a handful of queries per head (decode): one workgroup per head, its waves split the keys
     if (d->seq_q <= 32)
         return launch_attn_decode(a, d->head_dim, workspace, workspace_bytes, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
-    // 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per 256
-    // queries: a few % less energy, and this kernel is power-limited) when that still fills the chip: one
-    // workgroup per CU for unmasked attention; under a causal mask workgroups differ in length by up to
-    // n_qtiles x, so at least two rounds are needed to balance (measured at 512 wide workgroups: +2.3 % with head_dim 128, -10 % with 64, which is VALU- rather than power-bound).  Otherwise 4 waves x 32 (two workgroups per CU).
-#ifndef TRN_FORCE_NW
+    // Without score perturbation: the 16x16x32 kernel, in the workgroup shape its launcher's rule picks.
+    if (!noise)
+        return launch_attn_fwd16(a, d->head_dim, attn_fwd16_shape(d->batch, d->n_q_heads, d->seq_q, d->head_dim, d->causal != 0), s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
+    // With it: 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per
+    // 256 queries) when that still fills the chip -- one workgroup per CU for unmasked attention, two rounds under a
+    // causal mask, where workgroups differ in length; otherwise 4 waves x 32 (two workgroups per CU).
     const int64_t n_wide = (int64_t)((d->seq_q + 255) / 256) * d->batch * d->n_q_heads;
     const bool wide = n_wide >= (!d->causal ? 256 : d->head_dim == 128 ? 512 : 1024);
-#else
-    const bool wide = TRN_FORCE_NW == 8;
-#endif
-    // Without score perturbation: the 16x16x32 kernel; with head_dim 64 always its 4-wave form (measured: the 8-wave
-    // form loses 10-20 % there, at every size).
-    if (!noise) return launch_attn_fwd16(a, d->head_dim, wide && d->head_dim == 128, s) == hipSuccess ? TRN_OK : TRN_E_LAUNCH;
 #define TRN_LAUNCH(D_, NW_) launch_fwd<D_, NW_, true>(a, s)
     if (d->head_dim == 128) e = wide ? TRN_LAUNCH(128, 8) : TRN_LAUNCH(128, 4);
     else e = wide ? TRN_LAUNCH(64, 8) : TRN_LAUNCH(64, 4);

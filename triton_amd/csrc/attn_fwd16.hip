@@ -77,15 +77,29 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     const int BH = a.B * a.Hq;
-    const int qt = a.n_qtiles - 1 - (int)(blockIdx.x / BH);
     const int j = blockIdx.x % BH;
     const int G = a.Hq / a.Hkv, nkv = a.B * a.Hkv;
     const int kvslot = j % nkv, g = j / nkv;
     const int b = kvslot / a.Hkv, kvh = kvslot % a.Hkv, head = kvh * G + g;
 
     const int off = a.Skv - a.Sq;                       // causal: query i sees keys <= i + off
-    const int q0 = qt * BM;
-    const int wq0 = q0 + wave * 32;                     // first query of this wave
+    // Query rows.  Plain mode: the workgroup owns BM consecutive queries, latest (heaviest under a causal mask) tiles
+    // first.  Paired mode (NW = 8, causal, a grid too small for a second round to even out the tiles' lengths): waves
+    // 0-3 own the 128-query tile h, waves 4-7 the tile n - 1 - h from the other end, so that every workgroup has the
+    // same amount of work and each SIMD holds one long and one short wave.  K/V staging follows the later tile; the
+    // early waves stop at their own last visible tile as they do in plain mode.
+    int q0, q_last, wq0;
+    bool idle = false;
+    if (NW == 8 && a.paired) {
+        const int lt = (int)(blockIdx.x / BH), ht = a.n_qtiles - 1 - lt;     // n_qtiles counts 128-query tiles here
+        q0 = ht * 128; q_last = q0 + 127;
+        idle = wave >= 4 && lt == ht;                                       // odd tile count: the middle one is alone
+        wq0 = (wave < 4 ? ht : lt) * 128 + (wave & 3) * 32;
+        if (idle) wq0 = a.Sq;                                               // loads clamp, stores are predicated off
+    } else {
+        q0 = (a.n_qtiles - 1 - (int)(blockIdx.x / BH)) * BM; q_last = q0 + BM - 1;
+        wq0 = q0 + wave * 32;                           // first query of this wave
+    }
     int qrow[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) qrow[qb] = wq0 + 16 * qb + n;
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     float4_t lacc[2] = {zero, zero};
 
     int ntiles = (a.Skv + BN - 1) / BN;
-    if (a.causal) ntiles = min(ntiles, (min(q0 + BM - 1, a.Sq - 1) + off) / BN + 1);
+    if (a.causal) ntiles = min(ntiles, (min(q_last, a.Sq - 1) + off) / BN + 1);
 
     // ---- staging: direct global -> LDS loads; keys past the end read as zeros
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
@@ -338,6 +352,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     // others (its part of every refill, and the barrier), leaving its SIMD to the wave that still computes.
     int nlive = ntiles;
     if (a.causal) nlive = min(ntiles, (min(wq0 + 31, a.Sq - 1) + off) / BN + 1);
+    if (idle) nlive = 0;
     for (int jt = 0; jt < nlive; jt += 2) {
         tile(jt, Ks0, Ks1, Vs0, Vs1);
         if (jt + 1 < nlive) tile(jt + 1, Ks1, Ks0, Vs1, Vs0);
@@ -401,16 +416,48 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
 
 template <int D, int NW>
 static hipError_t launch16(AttnArgs a, hipStream_t s) {
-    a.n_qtiles = (a.Sq + 32 * NW - 1) / (32 * NW);
-    const int64_t grid = (int64_t)a.n_qtiles * a.B * a.Hq;
+    int64_t grid;
+    if (NW == 8 && a.paired) {
+        a.n_qtiles = (a.Sq + 127) / 128;
+        grid = (int64_t)((a.n_qtiles + 1) / 2) * a.B * a.Hq;
+    } else {
+        a.paired = 0;
+        a.n_qtiles = (a.Sq + 32 * NW - 1) / (32 * NW);
+        grid = (int64_t)a.n_qtiles * a.B * a.Hq;
+    }
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
     hipLaunchKernelGGL((attn_fwd16_kernel<D, NW>), dim3((unsigned)grid), dim3(NW * 64), 0, s, a);
     return hipGetLastError();
 }
 
-hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, bool wide, hipStream_t s) {
-    if (head_dim == 128) return wide ? launch16<128, 8>(a, s) : launch16<128, 4>(a, s);
-    return wide ? launch16<64, 8>(a, s) : launch16<64, 4>(a, s);
+// Workgroup shape by problem size.  Wide (each K/V stage is fetched from L2 once per 256 queries: a few % less energy,
+// and this kernel is power-limited) when that still fills the chip: one workgroup per CU for unmasked attention; under
+// a causal mask workgroups differ in length by up to n_qtiles x, so at least two rounds are needed to balance (measured
+// at 512 wide workgroups: +2.3 % with head_dim 128; with head_dim 64 the wide form loses 10-20 % at every size).  A
+// causal problem whose narrow workgroups would all be resident at once (a single round: the longest tile sets the time,
+// twice the mean) runs paired instead, which gives every workgroup the same work -- if the pairs still cover the chip.
+Attn16Shape attn_fwd16_shape(int batch, int n_q_heads, int seq_q, int head_dim, bool causal) {
+    const int64_t bh = (int64_t)batch * n_q_heads;
+    const int64_t n128 = (seq_q + 127) / 128;
+    // (paired workgroups are half as many: below about three quarters of the CUs the idle ones cost more than the
+    // imbalance -- measured at 1024 queries x 32 heads: 22.9 us narrow, 24.8 us paired; at 2048: 46.3 and 43.1)
+    if (causal && n128 * bh <= 512 && ((n128 + 1) / 2) * bh >= 192) return Attn16Shape::Paired;
+    const int64_t n_wide = (int64_t)((seq_q + 255) / 256) * bh;
+    return head_dim == 128 && n_wide >= (causal ? 512 : 256) ? Attn16Shape::Wide : Attn16Shape::Narrow;
+}
+
+hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, Attn16Shape shape, hipStream_t s) {
+    AttnArgs b = a;
+    b.paired = shape == Attn16Shape::Paired ? 1 : 0;
+    const bool wide = shape != Attn16Shape::Narrow;
+    if (head_dim == 128) return wide ? launch16<128, 8>(b, s) : launch16<128, 4>(b, s);
+    return wide ? launch16<64, 8>(b, s) : launch16<64, 4>(b, s);
+}
+
+const char* attn_fwd16_kernel_name(int head_dim, Attn16Shape shape) {
+    const bool wide = shape != Attn16Shape::Narrow;
+    if (head_dim == 128) return wide ? "trn::attn_fwd16_kernel<128, 8>" : "trn::attn_fwd16_kernel<128, 4>";
+    return wide ? "trn::attn_fwd16_kernel<64, 8>" : "trn::attn_fwd16_kernel<64, 4>";
 }
 
 }  // namespace trn
