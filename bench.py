@@ -47,11 +47,29 @@ def parse():
     return ap.parse_args()
 
 
-def graph_timed(module, tensors, steps, warmup, per_graph=20):
+CLOCK_WARMUP_S = 0.25      # untimed replays before any timed region: the board's clocks take tens of ms to settle
+REPEATS = 5                # the timed region (exactly `steps` forwards) is run this many times; the median is reported
+
+
+def _settle(replay, stream, seconds=CLOCK_WARMUP_S):
+    """Untimed replays until `seconds` of device work have run (a cold board is about 10 % slower for the first
+    30 ms of a burst than in steady state, and a single short timed region would measure mostly that)."""
+    import torch
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        with torch.cuda.stream(stream):
+            for _ in range(4):
+                replay()
+        stream.synchronize()
+
+
+def graph_timed(module, tensors, steps, warmup, per_graph=20, with_samples=False):
     """The reference driver's sequence -- cold call, warm-ups on a side stream, `forward` captured into a
     graph, replays -- except that one graph holds up to `per_graph` consecutive forwards, so that the gaps
     between graph launches (about as long as 5% of one attention kernel) stay out of the kernel timing.
-    Exactly `steps` forwards are timed.  Returns (wall ms/step, event ms/step)."""
+    A timed region is exactly `steps` forwards between device synchronisations; it is run REPEATS times after
+    the clocks have settled and the median region is reported.  Returns (wall ms/step, event ms/step)
+    [, the event ms/step of every region]."""
     import torch
     args = [tensors[p] for p in module.TENSOR_PARAMS]
     module.forward(*args)                       # cold call (allocates the module's workspaces)
@@ -71,24 +89,30 @@ def graph_timed(module, tensors, steps, warmup, per_graph=20):
                     module.forward(*args)
         graphs[n] = g
     stream.synchronize()
-    with torch.cuda.stream(stream):             # graph warm-up
-        graphs[sizes[0]].replay()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    with torch.cuda.stream(stream):
-        start.record()
-        for n in sizes:
-            graphs[n].replay()
-        end.record()
-    torch.cuda.synchronize()
-    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    return wall_ms, start.elapsed_time(end) / steps
+    _settle(graphs[sizes[0]].replay, stream)
+    regions = []
+    for _ in range(REPEATS):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(stream):
+            start.record()
+            for n in sizes:
+                graphs[n].replay()
+            end.record()
+        torch.cuda.synchronize()
+        regions.append(((time.perf_counter() - t0) * 1e3 / steps, start.elapsed_time(end) / steps))
+    regions_by_ev = sorted(regions, key=lambda r: r[1])
+    wall_ms, ev_ms = regions_by_ev[len(regions) // 2]
+    if with_samples:
+        return wall_ms, ev_ms, [r[1] for r in regions]
+    return wall_ms, ev_ms
 
 
 def rotating_timed(fn_for, n_buffers, steps, warmup):
     """One graph holding n_buffers launches, each on its own buffer set (so a launch never finds its data in
-    the last-level cache), replayed until `steps` launches have run; returns (wall ms/launch, event ms/launch).
+    the last-level cache), replayed until `steps` launches have run; REPEATS such regions after the clocks have
+    settled, the median reported; returns (wall ms/launch, event ms/launch).
     Capturing takes the Python call overhead -- longer than a 13 us kernel -- out of the timed region."""
     import torch
     stream = torch.cuda.Stream()
@@ -103,27 +127,30 @@ def rotating_timed(fn_for, n_buffers, steps, warmup):
                 fn_for(i)
     stream.synchronize()
     reps = max(1, (steps + n_buffers - 1) // n_buffers)
-    with torch.cuda.stream(stream):
-        graph.replay()
-    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    with torch.cuda.stream(stream):
-        start.record()
-        for _ in range(reps):
-            graph.replay()
-        end.record()
-    torch.cuda.synchronize()
+    _settle(graph.replay, stream, 0.1)
     n = reps * n_buffers
-    return (time.perf_counter() - t0) * 1e3 / n, start.elapsed_time(end) / n
+    regions = []
+    for _ in range(REPEATS):
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        with torch.cuda.stream(stream):
+            start.record()
+            for _ in range(reps):
+                graph.replay()
+            end.record()
+        torch.cuda.synchronize()
+        regions.append(((time.perf_counter() - t0) * 1e3 / n, start.elapsed_time(end) / n))
+    regions.sort(key=lambda r: r[1])
+    return regions[len(regions) // 2]
 
 
 def attn_inputs(cfg, seed=42):
     import torch
-    from oracle import ref
+    from triton_amd.configs import randn_half
     g = torch.Generator().manual_seed(seed)
     B, Hq, Hkv, S, D = cfg["batch"], cfg["n_heads"], cfg["n_kv_heads"], cfg["seq"], cfg["head_dim"]
-    q = ref.randn_half((B, Hq, S, D), g); k = ref.randn_half((B, Hkv, S, D), g); v = ref.randn_half((B, Hkv, S, D), g)
+    q = randn_half((B, Hq, S, D), g); k = randn_half((B, Hkv, S, D), g); v = randn_half((B, Hkv, S, D), g)
     return q, k, v
 
 
@@ -133,10 +160,12 @@ def bench_vanilla(steps, warmup):
     cfg = configs.VANILLA
     q, k, v = attn_inputs(cfg)
     t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda())
-    wall, ev = graph_timed(modules.get("vanilla"), t, steps, warmup)
+    wall, ev, samples = graph_timed(modules.get("vanilla"), t, steps, warmup, with_samples=True)
     flops = configs.attn_flops(cfg["batch"], cfg["n_heads"], cfg["seq"], cfg["seq"], cfg["head_dim"], True)
+    from triton_amd import ops
+    kernel = ops.attention_kernel_name(t["Q"], t["K"], t["V"], t["O"], cfg["head_dim"] ** -0.5, True)
     return dict(wall_ms=wall, kernel_ms=ev, flops=flops, tflops=flops / wall / 1e9, kernel_tflops=flops / ev / 1e9,
-                tensors=(q, k, v))
+                tensors=(q, k, v), kernel=kernel, region_ms=samples)
 
 
 def bench_rmsnorm(steps, warmup):
@@ -162,24 +191,24 @@ def bench_rmsnorm(steps, warmup):
 
 def bench_variant(name, steps, warmup):
     import torch
-    from oracle import ref
     from triton_amd import configs, modules
+    randn_half = configs.randn_half
     g = torch.Generator().manual_seed(42)
     if name == "qknorm":
         cfg = configs.QKNORM
         q, k, v = attn_inputs(cfg)
         D = cfg["head_dim"]
         t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda(),
-                 gamma_q=ref.randn_half((D,), g, 1, 0.02).cuda(), gamma_k=ref.randn_half((D,), g, 1, 0.02).cuda())
+                 gamma_q=randn_half((D,), g, 1, 0.02).cuda(), gamma_k=randn_half((D,), g, 1, 0.02).cuda())
         m = modules.get("qknorm", eps=cfg["eps"])
         flops = configs.attn_flops(1, cfg["n_heads"], cfg["seq"], cfg["seq"], D, True)
     elif name == "prenorm":
         cfg = configs.PRENORM
         S, N, D = cfg["seq"], cfg["hidden"], cfg["head_dim"]
         nkv = cfg["n_kv_heads"] * D
-        t = dict(X=ref.randn_half((1, S, N), g).cuda(), gamma=ref.randn_half((N,), g, 1, 0.02).cuda(),
-                 WQ=ref.randn_half((N, N), g, 0, 0.02).cuda(), WK=ref.randn_half((N, nkv), g, 0, 0.02).cuda(),
-                 WV=ref.randn_half((N, nkv), g, 0, 0.02).cuda(), O=torch.zeros(1, S, N, dtype=torch.float16, device="cuda"))
+        t = dict(X=randn_half((1, S, N), g).cuda(), gamma=randn_half((N,), g, 1, 0.02).cuda(),
+                 WQ=randn_half((N, N), g, 0, 0.02).cuda(), WK=randn_half((N, nkv), g, 0, 0.02).cuda(),
+                 WV=randn_half((N, nkv), g, 0, 0.02).cuda(), O=torch.zeros(1, S, N, dtype=torch.float16, device="cuda"))
         m = modules.get("prenorm", head_dim=D, eps=cfg["eps"])
         flops = configs.qkv_gemm_flops(S, N, N, nkv) + configs.attn_flops(1, cfg["n_heads"], S, S, D, True)
     elif name in ("keyformer", "roco"):
@@ -353,11 +382,15 @@ def main():
         "dtype": "f16", "data": "synthetic",
         "config": {"workload": "vanilla causal GQA attention, batch 1, seq 4096, 32 q heads / 8 kv heads, head_dim 128",
                    "flops_per_step": van["flops"], "flop_convention": "4*B*H*S^2*D/2 (causal-halved)",
-                   "timing": "graph replay on a side stream, 20 forwards per graph"},
+                   "timing": f"graph replay on a side stream, 20 forwards per graph; {CLOCK_WARMUP_S} s of untimed replays, "
+                             f"then {REPEATS} regions of exactly --steps forwards each, the median region reported"},
         "pct_of_fp16_mfma_peak": round(100 * van["tflops"] / peak, 2),
         "roofline": {"bound": "mfma", "achieved": round(van["kernel_tflops"], 2), "peak": peak, "unit": "TFLOP/s",
                      "frac": round(van["kernel_tflops"] / peak, 4), "traffic": traffic,
-                     "kernel": "trn::attn_fwd16_kernel<128, 8>", "kernel_ms": round(van["kernel_ms"], 5)},
+                     "kernel": van["kernel"], "kernel_ms": round(van["kernel_ms"], 5),
+                     "kernel_ms_per_region": [round(x, 5) for x in van["region_ms"]],
+                     "traffic_source": "profiles/attn_fwd_llama3_s4096_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
+                                       "WRITE_SIZE of this command, scaled by the library's copy kernel)"},
     }
     ceil = mfma_ceiling()
     line["roofline"]["mfma_only_kernel_tflops"] = {k: round(v, 1) for k, v in ceil.items()}

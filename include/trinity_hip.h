@@ -219,6 +219,14 @@ int trn_gate_f16(const void* c1, const void* c2, void* out, int64_t rows, int64_
                  int64_t ld1, int64_t ld2, int64_t ldo, int32_t kind, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: the name (as a profiler's kernel trace prints it) of the kernel
+ * instantiation that trn_attn_fwd_f16 launches for this problem -- decided by the same rules as the launch itself,
+ * so that a benchmark can say which kernel its timing belongs to.  with_noise: as if a noise tensor were passed.
+ * Returns "" for an invalid descriptor.  The string is static.
+ */
+const char* trn_attn_fwd_kernel_name(const trn_attn_desc* desc, int32_t with_noise);
+
+/*
  * Measurement aid, no counterpart in the reference: a plain 16-bytes-per-lane streaming copy of `bytes`
  * (a multiple of 16) from src to dst.  bench.py and the profiling recipes run it on a buffer of known size so
  * that HBM byte counters (FETCH_SIZE / WRITE_SIZE) and achieved GB/s of the real kernels can be scaled

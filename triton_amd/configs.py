@@ -34,3 +34,9 @@ def rmsnorm_bytes(rows: int, cols: int) -> int:
 
 def qkv_gemm_flops(tokens: int, hidden: int, n_q: int, n_kv: int) -> float:
     return 2.0 * tokens * hidden * (n_q + 2 * n_kv)
+
+
+def randn_half(shape, gen, mean: float = 0.0, std: float = 1.0):
+    """Synthetic fp16 tensor ~ N(mean, std) drawn in fp32 from a seeded generator (the benchmark inputs)."""
+    import torch
+    return (mean + std * torch.randn(shape, generator=gen, dtype=torch.float32)).half()

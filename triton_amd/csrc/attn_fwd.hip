@@ -412,10 +412,30 @@ int validate_attn(const trn_attn_desc* d, bool need_v) {
 
 }  // namespace trn
 
+namespace trn {
+// Workgroup shape of the forward kernel with score perturbation: 8 waves x 32 queries when that still fills the chip.
+static bool noise_kernel_wide(const trn_attn_desc* d) {
+    const int64_t n_wide = (int64_t)((d->seq_q + 255) / 256) * d->batch * d->n_q_heads;
+    return n_wide >= (!d->causal ? 256 : d->head_dim == 128 ? 512 : 1024);
+}
+}  // namespace trn
+
 extern "C" int64_t trn_attn_workspace_bytes(const trn_attn_desc* d) {
     using namespace trn;
     if (!d || validate_attn(d, true) != TRN_OK) return 0;
     return attn_decode_workspace_bytes(d->batch, d->n_q_heads, d->seq_q, d->seq_kv, d->head_dim);
+}
+
+extern "C" const char* trn_attn_fwd_kernel_name(const trn_attn_desc* d, int32_t with_noise) {
+    using namespace trn;
+    if (!d || validate_attn(d, true) != TRN_OK) return "";
+    const bool d128 = d->head_dim == 128;
+    if (d->seq_q <= 32) return with_noise ? (d128 ? "trn::attn_decode_kernel<128, true>" : "trn::attn_decode_kernel<64, true>")
+                                          : (d128 ? "trn::attn_decode_kernel<128, false>" : "trn::attn_decode_kernel<64, false>");
+    if (!with_noise) return attn_fwd16_kernel_name(d->head_dim, attn_fwd16_shape(d->batch, d->n_q_heads, d->seq_q, d->head_dim, d->causal != 0));
+    const bool wide = noise_kernel_wide(d);
+    if (d128) return wide ? "trn::attn_fwd_kernel<128, 8, true>" : "trn::attn_fwd_kernel<128, 4, true>";
+    return wide ? "trn::attn_fwd_kernel<64, 8, true>" : "trn::attn_fwd_kernel<64, 4, true>";
 }
 
 extern "C" int trn_attn_fwd_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
@@ -499,8 +519,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     // With it: 8 waves x 32 queries per workgroup (one workgroup per CU; each K/V stage is fetched from L2 once per
     // 256 queries) when that still fills the chip -- one workgroup per CU for unmasked attention, two rounds under a
     // causal mask, where workgroups differ in length; otherwise 4 waves x 32 (two workgroups per CU).
-    const int64_t n_wide = (int64_t)((d->seq_q + 255) / 256) * d->batch * d->n_q_heads;
-    const bool wide = n_wide >= (!d->causal ? 256 : d->head_dim == 128 ? 512 : 1024);
+    const bool wide = noise_kernel_wide(d);
 #define TRN_LAUNCH(D_, NW_) launch_fwd<D_, NW_, true>(a, s)
     if (d->head_dim == 128) e = wide ? TRN_LAUNCH(128, 8) : TRN_LAUNCH(128, 4);
     else e = wide ? TRN_LAUNCH(64, 8) : TRN_LAUNCH(64, 4);

@@ -139,6 +139,12 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
     _lib.check("trn_attn_fwd_f16", st)
 
 
+def attention_kernel_name(q, k, v, o, scale: float, causal: bool, with_noise: bool = False) -> str:
+    """Name of the kernel instantiation `attention` launches for these tensors, as a profiler prints it."""
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, None, 1.0)
+    return _lib.load().trn_attn_fwd_kernel_name(C.byref(d), 1 if with_noise else 0).decode()
+
+
 def attention_workspace_bytes(q, k, v, o, scale: float, causal: bool) -> int:
     """Bytes of workspace with which `attention` would split the keys of this problem over several workgroups (0: none)."""
     d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, None, 1.0)
