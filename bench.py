@@ -183,10 +183,14 @@ def bench_rmsnorm(steps, warmup):
     # the same footprint through a plain copy kernel: what a 1:1 read/write stream reaches on this machine
     from triton_amd import ops
     _, copy_ev = rotating_timed(lambda i: ops.calibration_copy(xs[i], ys[i]), R, max(steps, 64), warmup)
+    # ... and through a copy this build did not write: torch's Tensor.copy_ (device to device) on the same buffer pairs
+    _, tcopy_ev = rotating_timed(lambda i: ys[i].copy_(xs[i]), R, max(steps, 64), warmup)
     nbytes = configs.rmsnorm_bytes(cfg["rows"], cfg["cols"])
+    cbytes = 2 * cfg["rows"] * cfg["cols"] * 2
     return dict(kernel_us=ev * 1e3, gbps=nbytes / ev / 1e6, frac=nbytes / ev / 1e6 / configs.HBM_PEAK_GBPS,
                 hot_cache_gbps=nbytes / hot_ev / 1e6, bytes=nbytes, rotating_buffers=R,
-                copy_gbps=2 * cfg["rows"] * cfg["cols"] * 2 / copy_ev / 1e6)
+                copy_gbps=cbytes / copy_ev / 1e6, copy_us=copy_ev * 1e3,
+                torch_copy_gbps=cbytes / tcopy_ev / 1e6, torch_copy_us=tcopy_ev * 1e3)
 
 
 def bench_variant(name, steps, warmup):
@@ -401,6 +405,9 @@ def main():
                            "kernel_us": round(r["kernel_us"], 3), "bytes": r["bytes"],
                            "rotating_buffers": r["rotating_buffers"], "cache_hot_gbps": round(r["hot_cache_gbps"], 1),
                            "plain_copy_same_footprint_gbps": round(r["copy_gbps"], 1),
+                           "plain_copy_same_footprint_us": round(r["copy_us"], 3),
+                           "torch_copy_same_footprint_gbps": round(r["torch_copy_gbps"], 1),
+                           "torch_copy_same_footprint_us": round(r["torch_copy_us"], 3),
                            "workload": "RMSNorm fp16 [4096 x 4096], gamma, eps 1e-5"}
     for name in ("prenorm", "qknorm", "keyformer", "roco"):
         if name in extra:

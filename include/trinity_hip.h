@@ -64,7 +64,7 @@ int trn_check_device(void);
  *     row r -> outer = r / inner_rows, inner = r % inner_rows
  *     x + outer*x_outer_stride + (row_start + inner)*ldx ;  y likewise.
  * A plain [rows, cols] matrix is outer_rows = 1, inner_rows = rows, row_start = 0.
- * cols must be a multiple of 8 and <= 16384.
+ * cols must be a multiple of 8 and <= 16384.  y may be x itself (in place); gamma must not overlap y.
  */
 int trn_rmsnorm_f16(const void* x, const void* gamma /* nullable */, void* y,
                     int64_t outer_rows, int64_t inner_rows, int64_t cols,
@@ -87,7 +87,9 @@ typedef struct trn_attn_desc {
     int32_t q_norm;       /* 0 off, 1 on                                                   */
     float   q_norm_eps;
     /* KeyFormer perturbation (ref_rms.py:172): z = (scale*QK^T + noise) / tau.            */
-    int64_t noise_stride_b, noise_stride_h, noise_stride_s;   /* noise [b, hq, seq_q, seq_kv] float */
+    int64_t noise_stride_b, noise_stride_h, noise_stride_s;   /* noise [b, hq, seq_q, seq_kv] float; base and all
+                                                                 three pitches multiples of 16 bytes (seq_kv itself
+                                                                 may be anything: pad the rows)                   */
     float   tau;
 } trn_attn_desc;
 

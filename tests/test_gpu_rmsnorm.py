@@ -54,6 +54,20 @@ def test_head_rmsnorm_prefix_untouched():
     _check(out, want)
 
 
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (33, 520), (7, 16384)])
+def test_rmsnorm_in_place_equals_out_of_place(rows, cols):
+    """y may be x itself (DecodeQKNorm normalises the new cache rows where they lie): bit-identical to a separate y."""
+    from triton_amd import ops
+    g = torch.Generator().manual_seed(9)
+    x = ref.randn_half((rows, cols), g); gamma = ref.randn_half((cols,), g, 1.0, 0.02).cuda()
+    xd = x.cuda(); sep = torch.zeros_like(xd)
+    ops.rmsnorm(xd, gamma, sep, 1e-5)
+    ops.rmsnorm(xd, gamma, xd, 1e-5)
+    torch.cuda.synchronize()
+    assert torch.equal(xd, sep)
+    _check(xd, ref.rmsnorm(x, gamma.cpu(), 1e-5))
+
+
 def test_bad_arguments_raise():
     from triton_amd import ops, _lib
     x = torch.zeros(4, 12, dtype=torch.float16, device="cuda")

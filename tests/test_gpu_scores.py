@@ -70,6 +70,91 @@ def test_keyformer_parity(B, Hq, Hkv, Sq, Skv, D, causal, tau):
     assert torch.allclose(score.sum(-1).cpu(), torch.full((B, Hq), float(Sq)), rtol=1e-4)
 
 
+def _nan_padded(noise):
+    """fp32 device copy of `noise` whose rows are padded to a multiple of 4 floats, the padding filled with NaN."""
+    B, H, Sq, Skv = noise.shape
+    buf = torch.full((B, H, Sq, (Skv + 3) // 4 * 4), float("nan"), device="cuda")
+    view = buf[..., :Skv]
+    view.copy_(noise)
+    return view
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,tau", [
+    (1, 2, 1, 130, 257, 64, True, 1.0), (1, 2, 2, 203, 203, 128, True, 1.5), (1, 3, 1, 70, 198, 128, False, 1.0),   # prefill kernels
+    (1, 4, 2, 16, 1041, 128, False, 1.5), (2, 2, 2, 9, 702, 64, True, 1.0), (1, 3, 1, 32, 99, 128, True, 1.0)])     # decode kernel
+def test_keyformer_any_key_count_padding_never_read(B, Hq, Hkv, Sq, Skv, D, causal, tau):
+    """The reference's KeyFormer takes any cache length (ref_rms.py:147-179).  The kernels fetch noise 16 bytes at a
+    time, so its rows are padded to 4 floats; whatever the padding holds (NaN here) must never reach a sum."""
+    from triton_amd import ops
+    assert Skv % 4 != 0
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=21)
+    noise = ref.gumbel_noise((B, Hq, Sq, Skv), 77)
+    scale = D ** -0.5
+    qd, kd, vd, nd = q.cuda(), k.cuda(), v.cuda(), _nan_padded(noise)
+    o = torch.zeros_like(qd); lsep = torch.zeros(B, Hq, Sq, device="cuda"); score = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention_with_stats(qd, kd, vd, o, scale, causal, score, None, noise=nd, tau=tau, lse_pert=lsep)
+    torch.cuda.synchronize()
+    wo, wscore = ref.keyformer(q, k, v, noise, scale, tau, causal)
+    close_scores(score, wscore)
+    assert (o.float().cpu() - wo.float()).abs().max() < 2e-2
+    s = ref.scores_fp32(q, k, scale, causal)
+    assert torch.allclose(lsep.cpu(), torch.logsumexp((s + noise) / tau, -1), atol=1e-3, rtol=1e-3)
+
+
+def test_keyformer_split_keys_any_key_count():
+    from triton_amd import ops
+    B, Hq, Hkv, Sq, Skv, D, tau = 1, 8, 2, 16, 2067, 128, 1.5
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=22)
+    noise = ref.gumbel_noise((B, Hq, Sq, Skv), 78)
+    scale = D ** -0.5
+    qd, kd, vd, nd = q.cuda(), k.cuda(), v.cuda(), _nan_padded(noise)
+    o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda"); lsep = torch.zeros_like(lse)
+    n = ops.attention_workspace_bytes(qd, kd, vd, o, scale, False)
+    assert n > 0
+    ws = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, False, lse=lse, noise=nd, tau=tau, lse_pert=lsep, workspace=ws)
+    torch.cuda.synchronize()
+    s = ref.scores_fp32(q, k, scale, False)
+    assert torch.allclose(lsep.cpu(), torch.logsumexp((s + noise) / tau, -1), atol=1e-3, rtol=1e-3)
+    assert (o.float().cpu() - ref.attention(q, k, v, scale, False).float()).abs().max() < 2e-2
+
+
+@pytest.mark.parametrize("form,PM", [("decode", 1041), ("decode", 1042), ("prefill", 203)])
+def test_keyformer_modules_take_fp16_noise_of_any_length(form, PM):
+    """Through the module protocol with the reference's fp16 noise (convert_eval_rms.py:201) and a cache length that
+    is not a multiple of 4: the module pads its fp32 copy."""
+    from triton_amd import modules
+    g = torch.Generator().manual_seed(31)
+    if form == "decode":
+        M, N, D, H = 16, 512, 128, 4
+        P = PM - M
+        rnd = lambda *sh: (torch.randn(*sh, generator=g).clamp(-1, 1) * 0.05).half()
+        X, WQ, WK, WV = rnd(M, N), rnd(N, N), rnd(N, N), rnd(N, N)
+        Kc, Vc = rnd(H, PM, D), rnd(H, PM, D)
+        noise = torch.randn(H, M, PM, generator=g).half()
+        t = dict(X=X.cuda(), WQ=WQ.cuda(), WK=WK.cuda(), WV=WV.cuda(), K_cache=Kc.cuda(), V_cache=Vc.cuda(),
+                 O2=torch.zeros(M, N, dtype=torch.float16, device="cuda"), noise=noise.cuda(),
+                 C_out=torch.zeros(H, PM, dtype=torch.float16, device="cuda"))
+        m = modules.get("keyformer", "decode", head_dim=D)
+        m.forward(*[t[p] for p in m.TENSOR_PARAMS])
+        torch.cuda.synchronize()
+        wo, pw = ref.decode_append_keyformer(X, WQ, WK, WV, Kc, Vc, noise.float(), P, D, tau=1.5)
+        assert torch.allclose(t["O2"].float().cpu(), ref.flatten_token_major(wo).float(), atol=2e-2, rtol=1e-2)
+        close_scores(t["C_out"], pw.sum(1), rtol=2e-3, atol=1e-3)     # fp16 C_out: its own rounding on top of 1e-3
+    else:
+        B, Hq, Hkv, S, D = 1, 4, 2, PM, 64
+        q, k, v = make(B, Hq, Hkv, S, S, D, seed=32)
+        noise = ref.gumbel_noise((B, Hq, S, S), 79).half()
+        C_out = torch.zeros(B, Hq, S, device="cuda"); O = torch.zeros(B, Hq, S, D, dtype=torch.float16, device="cuda")
+        m = modules.get("keyformer", tau=1.0)
+        t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=O, noise=noise.cuda(), C_out=C_out)
+        m.forward(*[t[p] for p in m.TENSOR_PARAMS])
+        torch.cuda.synchronize()
+        wo, wc = ref.keyformer(q, k, v, noise.float(), D ** -0.5, 1.0, True)
+        close_scores(C_out, wc)
+        assert (O.float().cpu() - wo.float()).abs().max() < 2e-2
+
+
 def test_uniform_attention_harmonic_closed_form_on_gpu():
     S, D = 300, 128
     q, k, v = make(1, 2, 1, S, S, D, seed=3)

@@ -139,10 +139,15 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
                 s[r] = (key < a.Skv && (!a.causal || key <= qrow + off)) ? s[r] : -INFINITY;
             }
         }
-        if constexpr (NOISE) {          // row normaliser of z = (scale*s + g)/tau in the log2 domain (masked: -inf stays -inf)
+        if constexpr (NOISE) {          // row normaliser of z = (scale*s + g)/tau in the log2 domain
             float16_t z;
 #pragma unroll
             for (int r = 0; r < 16; ++r) z[r] = __builtin_fmaf(gc[r / 4][r % 4], a.c3, s[r] * a.c2);
+            if (masked) {               // a select, not arithmetic: what lies past a row's last key (the padding of
+                                        // the noise pitch) may be anything, NaN included
+#pragma unroll
+                for (int r = 0; r < 16; ++r) z[r] = s[r] == -INFINITY ? -INFINITY : z[r];
+            }
             const float zmax = fmaxf(m2, half_max(max16(z)));
             if (zmax > -INFINITY) {
                 float sum = 0.f;

@@ -8,7 +8,8 @@ namespace trn {
 // LPR lanes per row (power of two <= 64), NV 16-byte vectors per lane.
 template <int LPR, int NV>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(
-    const half_t* __restrict__ x, const half_t* __restrict__ gamma, half_t* __restrict__ y,
+    const half_t* x, const half_t* __restrict__ gamma, half_t* y,     // y may be x (in place): a row is read whole
+                                                                     // into registers before any of it is written
     int64_t n_rows, int64_t inner_rows, int cols,
     int64_t x_outer, int64_t ldx, int64_t y_outer, int64_t ldy, int64_t row_start, float eps) {
     constexpr int ROWS_PER_BLOCK = 256 / LPR;

@@ -86,6 +86,23 @@ def _scale(scale: Optional[float], head_dim: int) -> float:
     return head_dim ** -0.5 if scale is None else float(scale)
 
 
+def _noise_fp32(mod: "FusedModule", n4: torch.Tensor) -> torch.Tensor:
+    """The noise as the kernels read it: fp32, unit innermost stride, base and every pitch a multiple of 16 bytes
+    (they fetch it with 16-byte loads).  The reference's noise is fp16 (convert_eval_rms.py:201) and its key count
+    P + M is arbitrary, so anything else is copied into a workspace whose rows are padded to a multiple of 4 floats;
+    the padding is never read as a key (the kernels mask by key index, with selects)."""
+    ok = (n4.dtype == torch.float32 and n4.stride(3) == 1 and n4.data_ptr() % 16 == 0
+          and all(n4.stride(i) % 4 == 0 for i in range(3)))
+    if ok:
+        return n4
+    B, H, Sq, Skv = n4.shape
+    pitch = (Skv + 3) // 4 * 4
+    buf = mod._workspace("noise32", (B, H, Sq, pitch), torch.float32, n4.device)
+    view = buf[..., :Skv]
+    view.copy_(n4)
+    return view
+
+
 def _store_scores(dst: torch.Tensor, src32: torch.Tensor) -> None:
     """Key scores are produced in fp32; a caller-owned fp16 tensor (the reference allocates every
     tensor as fp16, vanilla_llama_benchmark.py:131-139) receives them rounded."""
@@ -154,11 +171,7 @@ class KeyFormerAttention(FusedModule):
         q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
         B, Hq, Sq, D = q.shape
         Skv = k.shape[2]
-        n4 = _as4(noise, "noise")
-        if n4.dtype != torch.float32:                    # the reference's noise is fp16 (convert_eval_rms.py:201)
-            n32 = self._workspace("noise32", n4.shape, torch.float32, n4.device)
-            n32.copy_(n4)
-            n4 = n32
+        n4 = _noise_fp32(self, _as4(noise, "noise"))
         lsep = self._workspace("lse_pert", (B, Hq, Sq), torch.float32, q.device)
         score = C_out.view(B, Hq, Skv) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
             self._workspace("score32", (B, Hq, Skv), torch.float32, q.device)
@@ -311,11 +324,7 @@ class DecodeKeyFormer(_DecodeAppend):
         q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
         H, M, D = q.shape
         PM = K_cache.shape[1]
-        n4 = noise[None]
-        if n4.dtype != torch.float32:
-            n32 = self._workspace("noise32", n4.shape, torch.float32, n4.device)
-            n32.copy_(n4)
-            n4 = n32
+        n4 = _noise_fp32(self, noise[None])
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
         score = C_out.view(1, H, PM) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
             self._workspace("score32", (1, H, PM), torch.float32, X.device)
