@@ -1,6 +1,7 @@
-"""GPU checks at the benchmarked (full) sizes: size-independent properties of the domain over the whole problem, and
-oracle parity on a sample of heads (the CPU oracle does one S=4096 head in a fraction of a second; all 32 would take
-minutes).  Tolerances as everywhere: fp16 attention outputs atol 2e-2 / rtol 1e-2, RMSNorm 1e-3 relative, fp32 key
+"""GPU checks at the benchmarked (full) sizes: oracle parity on every head of the problem (the CPU oracle does one
+S=4096 head in a few hundredths of a second), and size-independent properties of the domain over the whole problem.
+KeyFormer's noise is 2 GB for the whole problem; parity is taken on the four heads whose noise is drawn by the seeded
+host generator, the others (device-drawn noise) are held to the invariants.  Tolerances as everywhere: fp16 attention outputs atol 2e-2 / rtol 1e-2, RMSNorm 1e-3 relative, fp32 key
 scores 1e-3 relative."""
 import pytest
 import torch
@@ -32,7 +33,7 @@ def head_slice(q, k, v, h, group):
     return q[:, h:h + 1], k[:, h // group:h // group + 1], v[:, h // group:h // group + 1]
 
 
-def test_vanilla_llama_s4096_sampled_parity_and_properties():
+def test_vanilla_llama_s4096_parity_on_every_head_and_properties():
     from triton_amd import ops
     S = configs.VANILLA["seq"]; D = configs.LLAMA["head_dim"]; scale = D ** -0.5
     q, k, v = llama_qkv(S)
@@ -40,7 +41,7 @@ def test_vanilla_llama_s4096_sampled_parity_and_properties():
     o = torch.zeros_like(qd); lse = torch.zeros(1, 32, S, device="cuda")
     ops.attention(qd, kd, vd, o, scale, True, lse=lse)
     torch.cuda.synchronize()
-    for h in (0, 13, 31):                                   # first, a middle and the last query head
+    for h in range(32):
         wo, wl = ref.attention(*head_slice(q, k, v, h, 4), scale, True, return_lse=True)
         close(o[:, h:h + 1], wo); close(lse[:, h:h + 1], wl, atol=1e-3, rtol=1e-3)
     # a convex combination of V rows: constant V columns come back unchanged, whatever the weights
@@ -73,7 +74,7 @@ def test_vanilla_llama_s4096_sampled_parity_and_properties():
     close(o3[:, :, :t], o[:, :, :t])
 
 
-def test_roco_and_keyformer_llama_s4096_invariants_and_sampled_parity():
+def test_roco_and_keyformer_llama_s4096_invariants_and_parity():
     from triton_amd import ops
     S = configs.ROCO["seq"]; D = configs.LLAMA["head_dim"]; scale = D ** -0.5
     q, k, v = llama_qkv(S, seed=5)
@@ -87,11 +88,12 @@ def test_roco_and_keyformer_llama_s4096_invariants_and_sampled_parity():
     assert torch.allclose(s1.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
     assert (s2 >= 0).all() and (s2 <= s1 * (1 + 1e-5) + 1e-6).all()      # 0 <= p^2 <= p
     assert torch.isfinite(s1).all() and torch.isfinite(s2).all()
-    for h in (2, 30):
+    for h in range(32):
         qh, kh, vh = head_slice(q, k, v, h, 4)
         wo, w1, w2 = ref.roco(qh, kh, vh, scale, True)
         err1 = (s1[:, h:h + 1].cpu() - w1).abs(); err2 = (s2[:, h:h + 1].cpu() - w2).abs()
-        assert (err1 <= 1e-5 + 1e-3 * w1.abs()).all() and (err2 <= 1e-5 + 1e-3 * w2.abs()).all()
+        assert (err1 <= 1e-5 + 1e-3 * w1.abs()).all() and (err2 <= 1e-5 + 1e-3 * w2.abs()).all(), f"head {h}"
+        close(o[:, h:h + 1], wo)
     # KeyFormer with zero noise and tau = 1 is RoCo's column sum; with noise the scores still add up to S
     noise = torch.zeros(1, 32, S, S, device="cuda")
     lsep = torch.zeros(1, 32, S, device="cuda"); score = torch.full((1, 32, S), -1.0, device="cuda")
@@ -101,24 +103,27 @@ def test_roco_and_keyformer_llama_s4096_invariants_and_sampled_parity():
     # (the plain row sum is taken over the fp16-rounded probabilities that multiply V, the perturbed one in fp32)
     assert torch.allclose(lsep, lse, rtol=1e-3, atol=1e-3)
     assert torch.allclose(score, s1, rtol=1e-3, atol=1e-5)
-    # Gumbel noise drawn on the device for the whole problem (properties), from the seeded host generator for the
-    # sampled head (parity: both sides consume the same bits)
+    # Gumbel noise drawn on the device for the whole problem (properties), from the seeded host generator for four
+    # heads, one in each quarter (parity: both sides consume the same bits)
     u = torch.rand(1, 32, S, S, device="cuda").clamp_(1e-10, 1 - 1e-7)
     noise = -torch.log(-torch.log(u)); del u
-    h = 17
-    noise[:, h] = ref.gumbel_noise((1, 1, S, S), configs.KEYFORMER["noise_seed"])[:, 0].cuda()
+    heads = (1, 12, 17, 30)
+    host = ref.gumbel_noise((1, len(heads), S, S), configs.KEYFORMER["noise_seed"])
+    for i, h in enumerate(heads):
+        noise[:, h] = host[:, i].cuda()
     ops.attention(qd, kd, vd, o, scale, True, noise=noise, tau=1.0, lse_pert=lsep)
     ops.attention_colstats(qd, kd, lsep, scale, True, score, None, noise=noise, tau=1.0)
     torch.cuda.synchronize()
     assert torch.allclose(score.sum(-1).cpu(), torch.full((1, 32), float(S)), rtol=1e-4)
-    qh, kh, vh = head_slice(q, k, v, h, 4)
-    wo, wscore = ref.keyformer(qh, kh, vh, noise[:, h:h + 1].cpu(), scale, 1.0, True)
-    err = (score[:, h:h + 1].cpu() - wscore).abs()
-    assert (err <= 1e-5 + 1e-3 * wscore.abs()).all()
-    close(o[:, h:h + 1], wo)
+    for i, h in enumerate(heads):
+        qh, kh, vh = head_slice(q, k, v, h, 4)
+        wo, wscore = ref.keyformer(qh, kh, vh, host[:, i:i + 1], scale, 1.0, True)
+        err = (score[:, h:h + 1].cpu() - wscore).abs()
+        assert (err <= 1e-5 + 1e-3 * wscore.abs()).all(), f"head {h}"
+        close(o[:, h:h + 1], wo)
 
 
-def test_qknorm_falcon_s2048_sampled_parity_and_scale_invariance():
+def test_qknorm_falcon_s2048_parity_on_every_head_and_scale_invariance():
     from triton_amd import modules
     c = configs.QKNORM; S, H, D = c["seq"], c["n_heads"], c["head_dim"]
     g = torch.Generator().manual_seed(11)
@@ -135,7 +140,7 @@ def test_qknorm_falcon_s2048_sampled_parity_and_scale_invariance():
         return t["O"]
 
     o = run(q, k)
-    for h in (0, 35, 70):
+    for h in range(H):
         want = ref.qknorm_attention(q[:, h:h + 1], k, v, gq, gk, c["eps"], D ** -0.5, True)
         close(o[:, h:h + 1], want)
     # per-head RMSNorm makes the result (almost: eps) independent of the scale of Q and of K
@@ -143,7 +148,7 @@ def test_qknorm_falcon_s2048_sampled_parity_and_scale_invariance():
     close(o4, o, atol=2e-2)
 
 
-def test_prenorm_block_llama_s2048_sampled_parity():
+def test_prenorm_block_llama_s2048_parity_of_the_whole_output():
     from triton_amd import modules
     c = configs.PRENORM; S, N, D = c["seq"], c["hidden"], c["head_dim"]
     nkv = c["n_kv_heads"] * D

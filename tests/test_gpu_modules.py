@@ -127,11 +127,19 @@ def _decode_tensors(M, N, D, P, seed=42, amp=1.0):
     return {k: v.half() for k, v in t.items()}, H
 
 
+# a small problem, and the reference's own two (convert_eval_rms.py:33-60: Llama N=4096 H=32 D=128, Falcon N=4544
+# H=71 D=64; M=16 new tokens on a cache of P=1024)
+DECODE_SHAPES = [(16, 1024, 128, 200), (16, 4096, 128, 1024), (16, 4544, 64, 1024)]
+
+
+@pytest.mark.parametrize("M,N,D,P", DECODE_SHAPES)
 @pytest.mark.parametrize("amp", [1.0, 30.0])
-def test_decode_append_modules_match_reference_classes(amp):
-    """Reference-faithful mode: scale 1, no mask, MHA, M=16 new tokens on a P-token cache."""
+def test_decode_append_modules_match_reference_classes(amp, M, N, D, P):
+    """Reference-faithful mode: scale 1, no mask, MHA, M new tokens on a P-token cache; all five variants, whole
+    module outputs (O2, the appended cache rows, fp16 / fp32 key scores) against the CPU oracle."""
     from triton_amd import modules
-    M, N, D, P = 16, 1024, 128, 200
+    if amp > 1 and N > 1024:
+        amp = 30.0 * (1024 / N) ** 0.5       # keep the unscaled scores where they are at N = 1024 (they grow with N)
     cpu, H = _decode_tensors(M, N, D, P, amp=amp)
     W = (cpu["WQ"], cpu["WK"], cpu["WV"])
     atol = 2e-2 if amp > 1 else 1e-4
@@ -158,7 +166,10 @@ def test_decode_append_modules_match_reference_classes(amp):
         t[n] = (cpu[n] * wsc).half().cuda()
     Wp = tuple((w * wsc).half() for w in W)
     drive(modules.get("prenorm", "decode", head_dim=D), t, ["O2"])
-    close(t["O2"], ref.flatten_token_major(ref.decode_append_vanilla(cpu["X"], *Wp, cpu["K_cache"], cpu["V_cache"], P, D, prenorm=True)), atol)
+    # (with the norm, q and the new k are O(0.3) whatever the recipe's 0.01, and at N >= 4096 their one-ulp
+    # differences from the GEMM's summation order move O by up to 2e-3: the stated fp16 tolerance applies there)
+    close(t["O2"], ref.flatten_token_major(ref.decode_append_vanilla(cpu["X"], *Wp, cpu["K_cache"], cpu["V_cache"], P, D, prenorm=True)),
+          atol if N <= 1024 else 2e-2)
 
     t = fresh()
     drive(modules.get("qknorm", "decode", head_dim=D), t, ["O2"])

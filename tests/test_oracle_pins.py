@@ -236,6 +236,48 @@ def test_decode_append_vanilla_line_by_line():
     assert torch.equal(tm[:, D:2 * D], o[1])
 
 
+def test_decode_append_qknorm_brute_force_and_what_is_normalised():
+    """QKNorm.forward (ref_rms.py:205-229): q and the NEW k rows are divided by their root mean square over head_dim
+    (no eps, no weight), the cached prefix is used as stored, scores unscaled and unmasked.  Pinned by an fp64
+    loop-level definition, and by what the normalisation implies: the result does not change when W_q or W_k is
+    scaled, but does change when the cached prefix of K is (normalising the whole cache would hide that)."""
+    g = gen(17)
+    X, W, Kc, Vc, M, N, D, P, H = _decode_inputs(g)
+    o = ref.decode_append_qknorm(X, *W, Kc, Vc, P, D)
+    Xd = X.double().numpy(); Wd = [w.double().numpy() for w in W]
+    want = np.zeros((H, M, D))
+    for h in range(H):
+        # fp16-rounded projections, as the reference's half-precision matmul leaves them
+        q = np.array([[np.float16(sum(Xd[m, n] * Wd[0][n, h * D + d] for n in range(N))) for d in range(D)] for m in range(M)], dtype=np.float64)
+        k = np.array([[np.float16(sum(Xd[m, n] * Wd[1][n, h * D + d] for n in range(N))) for d in range(D)] for m in range(M)], dtype=np.float64)
+        v = np.array([[np.float16(sum(Xd[m, n] * Wd[2][n, h * D + d] for n in range(N))) for d in range(D)] for m in range(M)], dtype=np.float64)
+        for m in range(M):
+            qn = np.float16(q[m] / math.sqrt(sum(x * x for x in q[m]) / D)).astype(np.float64)
+            keys = [Kc[h, j].double().numpy() for j in range(P)]
+            vals = [Vc[h, j].double().numpy() for j in range(P)]
+            for j in range(M):
+                keys.append(np.float16(k[j] / math.sqrt(sum(x * x for x in k[j]) / D)).astype(np.float64))
+                vals.append(v[j])
+            s = [sum(qn[d] * kj[d] for d in range(D)) for kj in keys]
+            mx = max(s)
+            e = [math.exp(x - mx) for x in s]
+            z = sum(e)
+            for d in range(D):
+                want[h, m, d] = sum(e[j] * vals[j][d] for j in range(P + M)) / z
+    assert np.abs(o.double().numpy() - want).max() < 2e-3 * max(1.0, np.abs(want).max())
+    # invariant under the scale of W_q and of W_k (powers of two: exact in fp16) ...
+    o_q = ref.decode_append_qknorm(X, W[0] * 4, W[1], W[2], Kc, Vc, P, D)
+    o_k = ref.decode_append_qknorm(X, W[0], W[1] * 0.5, W[2], Kc, Vc, P, D)
+    assert torch.allclose(o_q.float(), o.float(), atol=2e-3) and torch.allclose(o_k.float(), o.float(), atol=2e-3)
+    # ... but not under the scale of the cached prefix, which is not normalised
+    Kc2 = Kc.clone(); Kc2[:, :P] *= 8
+    o_c = ref.decode_append_qknorm(X, *W, Kc2, Vc, P, D)
+    assert (o_c.float() - o.float()).abs().max() > 1e-2
+    # and the rows P.. of the cache that come in are ignored (they are overwritten by the new keys)
+    Kc3 = Kc.clone(); Kc3[:, P:] = 9.0
+    assert torch.equal(ref.decode_append_qknorm(X, *W, Kc3, Vc, P, D), o)
+
+
 def test_decode_append_variants_consistent():
     g = gen(16)
     X, W, Kc, Vc, M, N, D, P, H = _decode_inputs(g)
