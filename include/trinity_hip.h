@@ -161,6 +161,17 @@ int trn_attn_colstats_f16(const trn_attn_desc* desc, const void* q, const void* 
                           float* out_sum, float* out_sumsq, void* stream);
 
 /*
+ * RoCo's statistics as mean and standard deviation (BASELINE workload "per-key column mean and std of the attention
+ * probabilities"): out_mean[j] = (1/n_j) sum_i p_ij and out_std[j] = sqrt((1/n_j) sum_i p_ij^2 - out_mean[j]^2), the
+ * population standard deviation, over the n_j queries that can see key j (all seq_q of them without a mask;
+ * seq_q - max(0, j - (seq_kv - seq_q)) under a causal mask).  The reference defines the two sums only
+ * (ref_rms.py:274-275); these are formed from them in the same kernel's epilogue.  Arguments as
+ * trn_attn_colstats_f16 without noise; both outputs are required.
+ */
+int trn_attn_colmeanstd_f16(const trn_attn_desc* desc, const void* q, const void* k,
+                            const float* lse, float* out_mean, float* out_std, void* stream);
+
+/*
  * trn_attn_fwd_f16 and trn_attn_colstats_f16 in one call: the attention output plus the per-key statistics of its
  * probabilities -- of the perturbed probabilities when noise is given -- i.e. what one forward of the reference's
  * KeyFormer (ref_rms.py:147-179, C_out of keyformer_llama_benchmark.py:79) or RoCo (ref_rms.py:249-280) computes.
@@ -173,6 +184,18 @@ int trn_attn_fwd_stats_f16(const trn_attn_desc* desc, const void* q, const void*
                            void* o, float* lse, const void* gamma_q,
                            const float* noise, float* lse_pert,
                            float* out_sum, float* out_sumsq, void* stream);
+
+/*
+ * The decode-append form of KeyFormer as its reference class returns it (ref_rms.py:171-179): the attention output
+ * and the UN-REDUCED probabilities  out_probs[b,h,i,j] = softmax_j((scale*QK^T + noise)/tau)  (plain softmax(scale*QK^T)
+ * when noise is NULL), float [batch, n_q_heads, seq_q, seq_kv] contiguous, masked entries 0; optionally their sums
+ * over the queries as well (out_sum, nullable, as trn_attn_fwd_stats_f16).  One launch.  For decode shapes only:
+ * seq_q <= 32, otherwise TRN_E_UNSUPPORTED (at prefill sizes the matrix is what these kernels exist to avoid).
+ * lse / lse_pert as in trn_attn_fwd_f16 (lse_pert required with noise).
+ */
+int trn_attn_fwd_probs_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                           void* o, float* lse, const float* noise, float* lse_pert,
+                           float* out_probs, float* out_sum /* nullable */, void* stream);
 
 /*
  * Fused RMSNorm + Q/K/V projection:  Xn = RMSNorm(X; gamma, eps);  Q = Xn Wq, K = Xn Wk,

@@ -157,20 +157,9 @@ def test_module_protocol_host_logic():
     m = modules.get("vanilla")
     with pytest.raises(TypeError):
         m.forward(torch.zeros(1))                       # too few tensors
-    s1 = torch.tensor([[2.0, 1.0, 0.5]]); s2 = torch.tensor([[1.5, 0.6, 0.25]])
-    mean, std = modules.roco_mean_std(s1, s2, 3, True)
-    assert torch.allclose(mean, torch.tensor([[2 / 3, 0.5, 0.5]]))
-    assert torch.allclose(std, (s2 / torch.tensor([3.0, 2.0, 1.0]) - mean ** 2).clamp(min=0).sqrt())
-
-
-def test_roco_mean_std_matches_oracle_convention():
-    from oracle import ref
-    from triton_amd import modules
-    g = torch.Generator().manual_seed(0)
-    s1 = torch.rand(2, 3, 10, generator=g) + 0.5; s2 = s1 * 0.3
-    for causal, sq in ((True, 10), (True, 4), (False, 7)):
-        a = modules.roco_mean_std(s1, s2, sq, causal); b = ref.roco_mean_std(s1, s2, sq, causal)
-        assert torch.allclose(a[0], b[0]) and torch.allclose(a[1], b[1])
+    with pytest.raises(ValueError):
+        modules.get("roco", stats="variance")
+    assert modules.get("roco", stats="mean_std").TENSOR_PARAMS == modules.get("roco").TENSOR_PARAMS
 
 
 def test_bench_refuses_more_than_one_gpu():

@@ -78,9 +78,14 @@ def test_prefill_modules_under_graph_replay():
     drive(modules.get("roco"), t, ["O", "C_out1", "C_out2"])
     _, s1, s2 = ref.roco(q, k, v, scale, True)
     close(t["O"], want_o); close(t["C_out1"], s1, 1e-5, 1e-3); close(t["C_out2"], s2, 1e-5, 1e-3)
-    mean, std = modules.roco_mean_std(t["C_out1"], t["C_out2"], S, True)
-    wm, ws = ref.roco_mean_std(s1, s2, S, True)
-    close(mean, wm, 1e-6, 1e-3); close(std, ws, 1e-5, 5e-3)
+    # the same statistics as mean / standard deviation, from the kernel: against numpy over the visible rows of p
+    p = torch.softmax(ref.scores_fp32(q, k, scale, True).double(), -1).numpy()          # [B, Hq, S, S]
+    t2 = dict(t, C_out1=torch.zeros(B, Hq, S, device="cuda"), C_out2=torch.zeros(B, Hq, S, device="cuda"))
+    drive(modules.get("roco", stats="mean_std"), t2, ["O", "C_out1", "C_out2"])
+    for j in (0, 1, 17, 200, S - 2, S - 1):
+        col = p[0, :, j:, j]                                                             # queries i >= j see key j
+        close(t2["C_out1"][0, :, j], torch.from_numpy(col.mean(-1)), 1e-7, 1e-3)
+        close(t2["C_out2"][0, :, j], torch.from_numpy(col.std(-1)), 1e-6, 5e-3)
     # keyformer
     noise = ref.gumbel_noise((B, Hq, S, S), 1234)
     t = dict(Q=dev(q), K=dev(k), V=dev(v), O=torch.zeros_like(q).cuda(), noise=dev(noise),
@@ -189,6 +194,47 @@ def test_decode_append_modules_match_reference_classes(amp, M, N, D, P):
     # beyond the 1e-3 that holds for identical q,k (tests/test_gpu_scores.py) -- allow 5e-3 there.
     srt = 5e-3 if amp > 1 else 1e-3
     close(t["O2"], ref.flatten_token_major(wo), atol); close(t["C_out1"], s1, 1e-6, srt); close(t["C_out2"], s2, 1e-8, srt)
+
+
+@pytest.mark.parametrize("variant", ["vanilla", "qknorm", "roco"])
+def test_decode_append_head_major_placement_of_the_reference_classes(variant):
+    """ref_rms.py:80-81 views the head-major product [H,M,D] as [M,H*D] without transposing back; with
+    o_layout='head_major' O2's memory holds exactly that, so a swap-in against those classes compares equal."""
+    from triton_amd import modules
+    M, N, D, P = 16, 1024, 128, 200
+    cpu, H = _decode_tensors(M, N, D, P, amp=30.0)
+    W = (cpu["WQ"], cpu["WK"], cpu["WV"])
+    t = {k: v.cuda() for k, v in cpu.items()}
+    t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    t["C_out1"] = torch.zeros(H, P + M, device="cuda"); t["C_out2"] = torch.zeros(H, P + M, device="cuda")
+    m = modules.get(variant, "decode", head_dim=D, o_layout="head_major")
+    drive(m, t, ["O2"])
+    fn = {"vanilla": ref.decode_append_vanilla, "qknorm": ref.decode_append_qknorm,
+          "roco": lambda *a: ref.decode_append_roco(*a)[0]}[variant]
+    want = fn(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)                  # [H, M, D]
+    close(t["O2"], ref.flatten_head_major(want), 2e-2)
+    assert not torch.allclose(t["O2"].float().cpu(), ref.flatten_token_major(want).float(), atol=2e-2)
+    with pytest.raises(ValueError):
+        modules.get(variant, "decode", head_dim=D, o_layout="sideways")
+
+
+@pytest.mark.parametrize("M,N,D,P", [(16, 1024, 128, 200), (7, 512, 64, 333), (32, 512, 128, 1009)])
+def test_decode_keyformer_unreduced_perturb_out(M, N, D, P):
+    """KeyFormer.forward returns perturb_out [H,M,P+M] (ref_rms.py:174-179); reduce=False delivers it, fp32 or fp16."""
+    from triton_amd import modules
+    cpu, H = _decode_tensors(M, N, D, P, amp=10.0)
+    W = (cpu["WQ"], cpu["WK"], cpu["WV"])
+    wo, pw = ref.decode_append_keyformer(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], cpu["noise"], P, D, tau=1.5)
+    for dtype, rtol in ((torch.float32, 1e-2), (torch.float16, 1e-2)):
+        t = {k: v.cuda() for k, v in cpu.items()}
+        t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        t["C_out"] = torch.full((H, M, P + M), -1.0, dtype=dtype, device="cuda")
+        drive(modules.get("keyformer", "decode", head_dim=D, reduce=False), t, ["O2", "C_out"])
+        close(t["O2"], ref.flatten_token_major(wo), 2e-2)
+        # single probabilities, not sums: q and k come out of an fp16 GEMM whose summation order differs from the
+        # oracle's, and the unscaled softmax turns their one-ulp differences into up to 1 % of a probability
+        close(t["C_out"], pw, 1e-6, rtol)
+        assert torch.allclose(t["C_out"].float().sum(-1).cpu(), torch.ones(H, M), atol=2e-3)     # rows are distributions
 
 
 def test_first_call_inside_capture_is_refused():

@@ -155,6 +155,35 @@ def test_keyformer_modules_take_fp16_noise_of_any_length(form, PM):
         assert (O.float().cpu() - wo.float()).abs().max() < 2e-2
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", [(1, 2, 1, 40, 40, 64, True), (2, 4, 2, 33, 70, 128, True),
+                                                      (1, 3, 3, 50, 50, 64, False), (1, 2, 2, 130, 259, 128, True)])
+def test_roco_mean_and_std_from_the_kernel_against_numpy(B, Hq, Hkv, Sq, Skv, D, causal):
+    """trn_attn_colmeanstd_f16: per-key mean and standard deviation of the probabilities over the queries that see
+    the key, held to numpy's mean / std (population) of exactly those entries of the fp64 probability matrix."""
+    import numpy as np
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=13)
+    scale = D ** -0.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda")
+    mean = torch.full((B, Hq, Skv), -1.0, device="cuda"); std = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, causal, lse=lse)
+    ops.attention_col_mean_std(qd, kd, lse, scale, causal, mean, std)
+    torch.cuda.synchronize()
+    p = torch.softmax(ref.scores_fp32(q, k, scale, causal).double(), -1).numpy()
+    off = Skv - Sq
+    wm = np.zeros((B, Hq, Skv)); ws = np.zeros((B, Hq, Skv))
+    for j in range(Skv):
+        first = max(0, j - off) if causal else 0              # first query that sees key j
+        col = p[:, :, first:, j]
+        wm[:, :, j] = col.mean(-1); ws[:, :, j] = col.std(-1)
+    close_scores(mean, torch.from_numpy(wm), rtol=1e-3, atol=1e-7)
+    # sqrt(E p^2 - mean^2) in fp32 loses digits where the spread is far below the mean; such keys are held to 1e-3
+    # of the mean instead
+    err = (std.double().cpu() - torch.from_numpy(ws)).abs()
+    assert (err <= 2e-3 * torch.from_numpy(ws) + 1e-3 * torch.from_numpy(wm) + 1e-7).all()
+
+
 def test_uniform_attention_harmonic_closed_form_on_gpu():
     S, D = 300, 128
     q, k, v = make(1, 2, 1, S, S, D, seed=3)

@@ -168,6 +168,23 @@ def test_uniform_attention_harmonic_closed_forms():
     assert math.isclose(std[0, 0, j].item(), pj.std(unbiased=False).item(), rel_tol=1e-4)
 
 
+def test_roco_mean_std_is_numpy_mean_and_std_over_the_visible_rows():
+    """The convention of roco_mean_std, stated by what it must equal: numpy's mean and (population) std of column j of
+    the probability matrix, taken over the rows that can see key j."""
+    g = gen(21)
+    Sq, Skv = 9, 14
+    q, k, v = _qkv(g, 1, 2, 1, Sq, Skv, 8)
+    for causal in (True, False):
+        _, s1, s2 = ref.roco(q, k, v, 0.7, causal)
+        mean, std = ref.roco_mean_std(s1, s2, Sq, causal)
+        p = torch.softmax(ref.scores_fp32(q, k, 0.7, causal).double(), -1).numpy()
+        for j in range(Skv):
+            first = max(0, j - (Skv - Sq)) if causal else 0
+            col = p[0, :, first:, j]
+            assert np.allclose(mean[0, :, j].numpy(), col.mean(-1), rtol=1e-5)
+            assert np.allclose(std[0, :, j].numpy(), col.std(-1), rtol=1e-3, atol=1e-6)
+
+
 def test_tau_divides_both_score_and_noise():
     # (s + g)/tau, not s/tau + g and not s + g/tau: with tau=2 and doubled s, g it is the tau=1 result.
     g = gen(13)

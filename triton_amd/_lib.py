@@ -17,7 +17,7 @@ EXPORTS = (
     "trn_version", "trn_status_name", "trn_check_device", "trn_rmsnorm_f16",
     "trn_attn_fwd_f16", "trn_attn_colstats_f16", "trn_prenorm_qkv_f16", "trn_calibration_copy",
     "trn_calibration_mfma", "trn_attn_workspace_bytes", "trn_attn_fwd_ws_f16", "trn_linear_f16", "trn_gate_f16", "trn_attn_fwd_stats_f16",
-    "trn_attn_fwd_noalloc_f16", "trn_attn_fwd_kernel_name",
+    "trn_attn_fwd_noalloc_f16", "trn_attn_fwd_kernel_name", "trn_attn_colmeanstd_f16", "trn_attn_fwd_probs_f16",
 )
 
 
@@ -87,6 +87,10 @@ def load() -> C.CDLL:
     lib.trn_attn_fwd_kernel_name.argtypes = [C.POINTER(AttnDesc), C.c_int32]
     lib.trn_attn_colstats_f16.restype = C.c_int
     lib.trn_attn_colstats_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp]
+    lib.trn_attn_fwd_probs_f16.restype = C.c_int
+    lib.trn_attn_fwd_probs_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.trn_attn_colmeanstd_f16.restype = C.c_int
+    lib.trn_attn_colmeanstd_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp]
     lib.trn_prenorm_qkv_f16.restype = C.c_int
     lib.trn_prenorm_qkv_f16.argtypes = [vp] * 8 + [i64] * 15 + [f32, i32, vp]
     lib.trn_calibration_copy.restype = C.c_int

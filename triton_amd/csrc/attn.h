@@ -20,12 +20,14 @@ struct AttnArgs {
     // decode kernel only, one workgroup per head: per-key sums (and sums of squares) of the probabilities -- of the
     // perturbed ones when noise is given -- from a second sweep over the keys once the row normalisers are final
     float* col_sum; float* col_sumsq;
+    // ... and the probabilities themselves, un-reduced: float [B, Hq, Sq, Skv] contiguous
+    float* probs;
 };
 
 // Checks, argument block and kernel choice behind every attention entry point of the C ABI.
 int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
                  const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
-                 int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream);
+                 int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs = nullptr);
 
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream);

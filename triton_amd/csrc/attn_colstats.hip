@@ -33,6 +33,8 @@ struct ColArgs {
     float c1;   // log2-domain multiplier of the raw score: scale*log2e (RoCo) or scale*log2e/tau (KeyFormer)
     float c3;   // log2e/tau multiplier of the noise
     int causal;
+    int mean_std;   // write the per-key mean and population standard deviation over the queries that see the key
+                    // (into out_sum / out_sumsq) instead of the two sums
 };
 
 constexpr int CBN = 128;  // keys per workgroup
@@ -238,6 +240,13 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
 #pragma unroll
         for (int msk = 1; msk < 32; msk <<= 1) { x += __shfl_xor(x, msk, 64); if constexpr (SQ) y += __shfl_xor(y, msk, 64); }
         const int key = wkey0 + 8 * (r / 4) + 4 * h + (r % 4);
+        if (SQ && a.mean_std) {
+            // n = queries that see this key: all of them, or under a causal mask those from key - (Skv - Sq) on
+            const float n = (float)(a.causal ? a.Sq - max(0, key - (a.Skv - a.Sq)) : a.Sq);
+            const float mean = x / n;
+            y = __builtin_sqrtf(fmaxf(0.f, y / n - mean * mean));
+            x = mean;
+        }
         if (c == 0 && key < a.Skv) {
             if (a.out_sum) a.out_sum[obase + key] = x;
             if (SQ && a.out_sumsq) a.out_sumsq[obase + key] = y;
@@ -256,9 +265,24 @@ static hipError_t launch_col(const ColArgs& a, hipStream_t s) {
 
 }  // namespace trn
 
+namespace trn {
+static int colstats(const trn_attn_desc* d, const void* q, const void* k, const float* lse, const float* noise,
+                    float* out_sum, float* out_sumsq, int mean_std, void* stream);
+}
+
 extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, const void* k, const float* lse,
                                      const float* noise, float* out_sum, float* out_sumsq, void* stream) {
-    using namespace trn;
+    return trn::colstats(d, q, k, lse, noise, out_sum, out_sumsq, 0, stream);
+}
+
+extern "C" int trn_attn_colmeanstd_f16(const trn_attn_desc* d, const void* q, const void* k, const float* lse,
+                                       float* out_mean, float* out_std, void* stream) {
+    if (!out_mean || !out_std) return TRN_E_NULL;
+    return trn::colstats(d, q, k, lse, nullptr, out_mean, out_std, 1, stream);
+}
+
+static int trn::colstats(const trn_attn_desc* d, const void* q, const void* k, const float* lse, const float* noise,
+                         float* out_sum, float* out_sumsq, int mean_std, void* stream) {
     if (!d || !q || !k || !lse) return TRN_E_NULL;
     if (!out_sum && !out_sumsq) return TRN_E_NULL;
     int st = validate_attn(d, false);
@@ -288,6 +312,7 @@ extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, cons
     const float tau = noise ? d->tau : 1.f;
     a.c1 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.causal = d->causal ? 1 : 0;
+    a.mean_std = mean_std;
     if ((int64_t)a.n_kvtiles * a.B * a.Hq > 0x7fffffffLL) return TRN_E_SHAPE;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;

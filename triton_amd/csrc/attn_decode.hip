@@ -365,7 +365,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     // register operands with their roles swapped -- so that a lane owns one KEY and holds 16 of the 32 queries: the
     // sum over queries is in-lane plus one exchange with lane^32, and a block's 32 sums are one 128-byte store.
     // (Only with one workgroup per head: the launcher does not split the keys when these outputs are asked for.)
-    if (a.col_sum || a.col_sumsq) {
+    if (a.col_sum || a.col_sumsq || a.probs) {
         __syncthreads();                                   // every thread has read the merge arrays
         if (dg == 0) st_l[0][q] = NOISE ? ms2 + fast_log2(L2) : mstar + fast_log2(L);     // log2 domain
         __syncthreads();
@@ -405,6 +405,8 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
                 if constexpr (NOISE) t = __builtin_fmaf(gc[r], a.c3, t);
                 const bool ok = key < a.Skv && qr < a.Sq && (!a.causal || key <= qr + off);
                 const float p = ok ? fast_exp2(t) : 0.f;
+                // (32 consecutive keys of one query row per store instruction: whole 128-byte lines)
+                if (a.probs && key < a.Skv && qr < a.Sq) a.probs[((int64_t)bh * a.Sq + qr) * a.Skv + key] = p;
                 x += p;
                 y = __builtin_fmaf(p, p, y);
             }
@@ -449,7 +451,7 @@ int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     a.n_split = 1; a.ws = nullptr;
     const int64_t need = attn_decode_workspace_bytes(a.B, a.Hq, a.Sq, a.Skv, head_dim);
-    if (workspace && need > 0 && workspace_bytes >= need && !a.col_sum && !a.col_sumsq) {
+    if (workspace && need > 0 && workspace_bytes >= need && !a.col_sum && !a.col_sumsq && !a.probs) {
         a.n_split = decode_splits(a.B, a.Hq, a.Skv, head_dim);
         a.ws = static_cast<float*>(workspace);
     }

@@ -453,6 +453,16 @@ extern "C" int trn_attn_fwd_ws_f16(const trn_attn_desc* d, const void* q, const 
 extern "C" int trn_attn_colstats_f16(const trn_attn_desc* d, const void* q, const void* k, const float* lse,
                                      const float* noise, float* out_sum, float* out_sumsq, void* stream);
 
+extern "C" int trn_attn_fwd_probs_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                      float* lse, const float* noise, float* lse_pert,
+                                      float* out_probs, float* out_sum, void* stream) {
+    using namespace trn;
+    if (!d || !out_probs) return TRN_E_NULL;
+    if (d->seq_q > 32) return TRN_E_UNSUPPORTED;     // the un-reduced matrix is a decode-shape output
+    if (d->q_norm) return TRN_E_UNSUPPORTED;
+    return attn_forward(d, q, k, v, o, lse, nullptr, noise, lse_pert, nullptr, 0, out_sum, nullptr, stream, out_probs);
+}
+
 extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
                                       float* lse, const void* gamma_q, const float* noise, float* lse_pert,
                                       float* out_sum, float* out_sumsq, void* stream) {
@@ -472,7 +482,7 @@ extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, con
 
 int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
                              const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
-                             int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream) {
+                             int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs) {
     if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;
     if (!d || !q || !k || !v || !o) return TRN_E_NULL;
     if (noise && !lse_pert) return TRN_E_NULL;
@@ -503,7 +513,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
-    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.paired = 0;
+    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs; a.paired = 0;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
     if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)

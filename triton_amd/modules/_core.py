@@ -182,13 +182,17 @@ class KeyFormerAttention(FusedModule):
 
 
 class RoCoAttention(FusedModule):
-    """Attention plus per-key column sum C_out1 and column sum of squares C_out2 of the attention
-    probabilities (ref_rms.py:274-275).  mean/std are derived by roco_mean_std below."""
+    """Attention plus per-key statistics of the attention probabilities.  stats='sums' (the reference's form,
+    ref_rms.py:274-275): C_out1 = column sum, C_out2 = column sum of squares.  stats='mean_std': C_out1 = mean and
+    C_out2 = population standard deviation over the queries that can see the key, formed from the two sums in the
+    statistics kernel's epilogue."""
     TENSOR_PARAMS = ["C_out1", "C_out2", "K", "O", "Q", "V"]
 
-    def __init__(self, scale: Optional[float] = None, causal: bool = True):
+    def __init__(self, scale: Optional[float] = None, causal: bool = True, stats: str = "sums"):
         super().__init__()
-        self.scale, self.causal = scale, causal
+        if stats not in ("sums", "mean_std"):
+            raise ValueError("stats: expected 'sums' or 'mean_std'")
+        self.scale, self.causal, self.stats = scale, causal, stats
 
     def _run(self, C_out1, C_out2, K, O, Q, V):
         q, k, v, o = _as4(Q, "Q"), _as4(K, "K"), _as4(V, "V"), _as4(O, "O")
@@ -201,23 +205,11 @@ class RoCoAttention(FusedModule):
                         self._workspace(f"stat32_{i}", (B, Hq, Skv), torch.float32, q.device))
         sc = _scale(self.scale, D)
         ops.attention(q, k, v, o, sc, self.causal, lse=lse)
-        ops.attention_colstats(q, k, lse, sc, self.causal, outs[0], outs[1])
+        if self.stats == "sums":
+            ops.attention_colstats(q, k, lse, sc, self.causal, outs[0], outs[1])
+        else:
+            ops.attention_col_mean_std(q, k, lse, sc, self.causal, outs[0], outs[1])
         _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
-
-
-def roco_mean_std(s1: torch.Tensor, s2: torch.Tensor, seq_q: int, causal: bool):
-    """Per-key mean and (population) standard deviation of the attention probabilities over the
-    queries that can see the key, from RoCo's two sums.  n_j = seq_q - max(0, j - (seq_kv - seq_q))
-    under a causal mask, seq_q otherwise.  The reference defines only the sums; this derived
-    convention is this build's own."""
-    skv = s1.shape[-1]
-    if causal:
-        j = torch.arange(skv, device=s1.device)
-        n = (seq_q - (j - (skv - seq_q)).clamp(min=0)).to(s1.dtype)
-    else:
-        n = torch.full((skv,), float(seq_q), device=s1.device, dtype=s1.dtype)
-    mean = s1 / n
-    return mean, (s2 / n - mean * mean).clamp(min=0).sqrt()
 
 
 class PreNormBlock(FusedModule):
@@ -253,11 +245,16 @@ class _DecodeAppend(FusedModule):
     """Common part of the reference's own problem form (ref_rms.py:45-83): M new tokens X [M,N] are
     projected with WQ/WK/WV [N,N]; K and V rows are appended in place at rows P..P+M of the
     [H,P+M,D] caches (convert_eval_rms.py:146-147); every query then attends to all P+M keys with
-    no mask and no scale; O2 [M,N] is token-major (convert_eval_rms.py:160)."""
+    no mask and no scale.  O2 [M,N]: o_layout='token_major' puts head h of token m at O2[m, h*D:(h+1)*D], as the
+    generated kernels do (convert_eval_rms.py:160); 'head_major' fills O2's memory as [H,M,D], which is what the
+    reference classes' `output.view(M, H*D)` of the head-major product leaves there (ref_rms.py:80-81)."""
 
-    def __init__(self, head_dim: int, prenorm: bool = False, scale: float = 1.0, causal: bool = False):
+    def __init__(self, head_dim: int, prenorm: bool = False, scale: float = 1.0, causal: bool = False,
+                 o_layout: str = "token_major"):
         super().__init__()
-        self.head_dim, self.prenorm, self.scale, self.causal = head_dim, prenorm, scale, causal
+        if o_layout not in ("token_major", "head_major"):
+            raise ValueError("o_layout: expected 'token_major' or 'head_major'")
+        self.head_dim, self.prenorm, self.scale, self.causal, self.o_layout = head_dim, prenorm, scale, causal, o_layout
 
     def _project(self, X, WQ, WK, WV, K_cache, V_cache):
         M, N = X.shape
@@ -270,9 +267,11 @@ class _DecodeAppend(FusedModule):
         ops.prenorm_qkv(X, None, WQ, WK, WV, q, K_cache[:, P:], V_cache[:, P:], 0.0, self.prenorm)
         return q, P
 
-    @staticmethod
-    def _o_view(O2, H, M, D):
-        return O2.view(M, H, D).permute(1, 0, 2).unsqueeze(0)               # [1,H,M,D] view of token-major O2
+    def _o_view(self, O2, H, M, D):
+        """[1,H,M,D] view of O2's memory in the module's output placement."""
+        if self.o_layout == "head_major":
+            return O2.view(H, M, D).unsqueeze(0)
+        return O2.view(M, H, D).permute(1, 0, 2).unsqueeze(0)
 
     def _attend(self, q, K_cache, V_cache, O2, **kw):
         """Attention of the M new queries over the whole cache, with a workspace (allocated and zeroed once per shape;
@@ -312,13 +311,14 @@ class DecodeQKNorm(_DecodeAppend):
 
 
 class DecodeKeyFormer(_DecodeAppend):
-    """KeyFormer.forward (ref_rms.py:147-179) with the perturbed probabilities summed over the M
-    queries into C_out [H,P+M] as the generated kernel does (keyformer_llama_benchmark.py:79)."""
+    """KeyFormer.forward (ref_rms.py:147-179).  reduce=True: the perturbed probabilities summed over the M queries
+    into C_out [H,P+M] as the generated kernel does (keyformer_llama_benchmark.py:79).  reduce=False: C_out is the
+    un-reduced perturb_out [H,M,P+M] that the reference class returns (ref_rms.py:174-179); M <= 32."""
     TENSOR_PARAMS = ["C_out", "K_cache", "O2", "V_cache", "WK", "WQ", "WV", "X", "noise"]
 
-    def __init__(self, head_dim: int, tau: float = 1.5, **kw):
+    def __init__(self, head_dim: int, tau: float = 1.5, reduce: bool = True, **kw):
         super().__init__(head_dim, **kw)
-        self.tau = tau
+        self.tau, self.reduce = tau, reduce
 
     def _run(self, C_out, K_cache, O2, V_cache, WK, WQ, WV, X, noise):
         q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
@@ -326,11 +326,19 @@ class DecodeKeyFormer(_DecodeAppend):
         PM = K_cache.shape[1]
         n4 = _noise_fp32(self, noise[None])
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
-        score = C_out.view(1, H, PM) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
-            self._workspace("score32", (1, H, PM), torch.float32, X.device)
-        # one launch up to 32 new tokens (the key scores are a second sweep inside the attention kernel), two beyond
-        ops.attention_with_stats(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
-                                 score, None, noise=n4, tau=self.tau, lse_pert=lsep)
+        shape = (1, H, PM) if self.reduce else (1, H, M, PM)
+        if C_out.numel() != H * PM * (1 if self.reduce else M):
+            raise ValueError(f"C_out {tuple(C_out.shape)}: expected {shape[1:]}")
+        score = C_out.view(shape) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
+            self._workspace("score32", shape, torch.float32, X.device)
+        o = self._o_view(O2, H, M, D)
+        if self.reduce:
+            # one launch up to 32 new tokens (the key scores are a second sweep inside the attention kernel), two beyond
+            ops.attention_with_stats(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
+                                     score, None, noise=n4, tau=self.tau, lse_pert=lsep)
+        else:
+            ops.attention_with_probs(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
+                                     score, noise=n4, tau=self.tau, lse_pert=lsep)
         _store_scores(C_out, score)
 
 

@@ -170,6 +170,37 @@ def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[
     _lib.check("trn_attn_colstats_f16", st)
 
 
+def attention_with_probs(q, k, v, o, scale: float, causal: bool, out_probs: torch.Tensor,
+                         out_sum: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                         noise: Optional[torch.Tensor] = None, tau: float = 1.0,
+                         lse_pert: Optional[torch.Tensor] = None) -> None:
+    """Decode shapes (at most 32 queries per head): o, and the un-reduced probabilities out_probs float32
+    [B,Hq,Sq,Skv] -- of the perturbed scores when noise is given (KeyFormer's perturb_out) -- in one launch."""
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, noise, tau)
+    B, Hq, Sq, _ = q.shape
+    Skv = k.shape[2]
+    _dev_float(out_probs, "out_probs")
+    _need(tuple(out_probs.shape) == (B, Hq, Sq, Skv) and out_probs.is_contiguous(), f"out_probs: expected contiguous float32 {(B, Hq, Sq, Skv)}")
+    _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq)); _row_stat(out_sum, "out_sum", (B, Hq, Skv))
+    _need(noise is None or lse_pert is not None, "noise requires lse_pert")
+    st = _lib.load().trn_attn_fwd_probs_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(noise),
+                                            _ptr(lse_pert), _ptr(out_probs), _ptr(out_sum), _stream(q))
+    _lib.check("trn_attn_fwd_probs_f16", st)
+
+
+def attention_col_mean_std(q, k, lse, scale: float, causal: bool, out_mean: torch.Tensor, out_std: torch.Tensor) -> None:
+    """Per-key mean and population standard deviation of the attention probabilities exp(scale*q k^T - lse) over the
+    queries that can see the key (RoCo's statistics in that form).  out_mean, out_std: float32 [B,Hq,Skv]."""
+    d = _attn_desc(q, k, None, None, scale, causal, False, 0.0, None, 1.0)
+    B, Hq, Sq, _ = q.shape
+    Skv = k.shape[2]
+    _need(lse is not None and out_mean is not None and out_std is not None, "lse, out_mean and out_std are required")
+    _row_stat(lse, "lse", (B, Hq, Sq))
+    _row_stat(out_mean, "out_mean", (B, Hq, Skv)); _row_stat(out_std, "out_std", (B, Hq, Skv))
+    st = _lib.load().trn_attn_colmeanstd_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(lse), _ptr(out_mean), _ptr(out_std), _stream(q))
+    _lib.check("trn_attn_colmeanstd_f16", st)
+
+
 def attention_with_stats(q, k, v, o, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
                          out_sumsq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                          noise: Optional[torch.Tensor] = None, tau: float = 1.0,
