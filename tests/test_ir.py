@@ -147,6 +147,54 @@ def test_candidates_are_recognised(variant, index):
 def test_lora_and_gated_mlp_candidates_are_recognised(variant, index):
     m = ir.recognise(LINEAR[variant][index])
     assert m.variant == variant, m.reason
+    if variant == "gmlp":
+        # the first candidate gates with sigmoid(X W1); the second computes C1 C2 / (1 + exp(-C1)) = SiLU(C1) C2
+        assert m.kwargs == {"gate": ("sigmoid", "silu")[index]}
+    else:
+        assert m.kwargs == {}
+
+
+def test_keyformer_temperature_is_read_off_the_candidate():
+    """The module is built with the divisor the candidate applies to its perturbed scores (ref_rms.py:172 divides by
+    1.5); a candidate with another constant gets that one, one without a division gets 1, and a divisor that is not a
+    number is not something the hand-written module can be built for."""
+    c = CANDIDATES["keyformer"][0]
+    assert ir.recognise(c).kwargs == {"tau": 1.5}
+    assert ir.recognise(c.replace("noise) (index (elem h) fulltile (tile p)))) 1.5))", "noise) (index (elem h) fulltile (tile p)))) 2))")).kwargs == {"tau": 2.0}
+    no_div = c.replace("(exp (/ (+ ", "(exp (+ ").replace("(load (input noise) (index (elem h) fulltile (tile p)))) 1.5))", "(load (input noise) (index (elem h) fulltile (tile p)))))")
+    m = ir.recognise(no_div)
+    assert m.variant == "keyformer" and m.kwargs == {"tau": 1.0}, m.reason
+    m = ir.recognise(c.replace("(tile p)))) 1.5))", "(tile p)))) T))"))
+    assert not m and "temperature" in m.reason
+
+
+def _tree(n):
+    """ir.Node -> nested tuples, so that the expected trees below can be written as plain literals."""
+    return (n.op, *(_tree(a) for a in n.args)) if isinstance(n, ir.Node) else n
+
+
+def test_parse_against_trees_written_out_by_hand_from_the_reference_parser():
+    """What IrParser.parse builds for the constructs that have code of their own there, written out by hand
+    (a VAR child of the reference is a bare string here, a NUM child an int, other nodes (op, children...))."""
+    # names under input / output / tensor: a comma-separated list becomes one VAR child per name, in order
+    # (IrParser.py:63-87); spaces around the commas do not matter (the tokenizer splits on them, :13-19)
+    assert _tree(ir.parse("(input X,Y)")) == ("input", "X", "Y")
+    assert _tree(ir.parse("(output A , B)")) == ("output", "A", "B")
+    assert _tree(ir.parse("(tensor C_exp, C_sum ,C_div)")) == ("tensor", "C_exp", "C_sum", "C_div")
+    # a single name is parsed as an ordinary expression: one VAR child (IrParser.py:88-91)
+    assert _tree(ir.parse("(input X)")) == ("input", "X")
+    # `fulltile` and `dummy` are nodes without children whether bare (IrParser.py:44-49) or parenthesised (:107, :123)
+    assert _tree(ir.parse("(index fulltile (fulltile) (tile n))")) == ("index", ("fulltile",), ("fulltile",), ("tile", "n"))
+    assert _tree(ir.parse("(seq dummy (dummy))")) == ("seq", ("dummy",), ("dummy",))
+    # integers, negative ones included, are NUM; anything else bare is a VAR, also `P+M` and `1.5` (IrParser.py:38-40, :50-51)
+    assert _tree(ir.parse("(const_tile P+M -16)")) == ("const_tile", "P+M", -16)
+    assert _tree(ir.parse("(/ x 1.5)")) == ("/", "x", "1.5")
+    # a whole statement: store of two outputs from a load of two inputs
+    got = _tree(ir.parse("(sloop 0 P+M 16 p (store (output A, B) (x (load (input X,Y) (index (tile p) fulltile)) 2) (index (elem h) (tile p))))"))
+    assert got == ("sloop", 0, "P+M", 16, "p",
+                   ("store", ("output", "A", "B"),
+                    ("x", ("load", ("input", "X", "Y"), ("index", ("tile", "p"), ("fulltile",))), 2),
+                    ("index", ("elem", "h"), ("tile", "p"))))
 
 
 @pytest.mark.parametrize("name", UNSUPPORTED)
@@ -199,10 +247,11 @@ def ir_file(tmp_path):
 def test_candidates_of_a_file_are_selected_like_the_reference_flags(tmp_path):
     from triton_amd import benchmark
     path = ir_file(tmp_path)
-    assert [(i, v) for i, _, v, _ in benchmark.candidates_from_ir(path, 0, None)] == \
+    assert [(i, v) for i, _, v, *_ in benchmark.candidates_from_ir(path, 0, None)] == \
         [(0, "vanilla"), (1, "roco"), (2, None), (3, "keyformer"), (4, "qknorm")]
     assert [i for i, *_ in benchmark.candidates_from_ir(path, 1, 2)] == [1, 2]
     assert [i for i, *_ in benchmark.candidates_from_ir(path, 3, 10)] == [3, 4]
+    assert benchmark.candidates_from_ir(path, 3, 1)[0][4] == {"tau": 1.5}          # constants read off the candidate
 
 
 def test_evaluate_checks_the_case_file_against_the_variant(tmp_path, capsys):
@@ -229,6 +278,70 @@ def test_benchmark_cli_times_recognised_candidates_and_records_the_rest(tmp_path
     assert all(d["error"] is None and 0 < d["execution_time_ms"] < 10 for d in data if d["ir_id"] != 2)
     assert data[2]["error"].startswith("unsupported IR") and math.isinf(data[2]["execution_time_ms"])
     assert data[0]["ir_expression"].startswith("(seq (ploop")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("variant,index", [(v, i) for table in (CANDIDATES, LINEAR) for v, c in table.items() for i in range(len(c))])
+def test_recognised_candidate_runs_and_matches_the_oracle(variant, index):
+    """parse -> recognise -> module -> run, as the reference's drivers go from a candidate to a timed module
+    (vanilla_llama_benchmark.py:141-221): the module a candidate is mapped to, built with the constants read off the
+    candidate, computes what the oracle says that workload computes."""
+    import torch
+    from oracle import ref
+    from triton_amd import modules
+    m = ir.recognise((CANDIDATES.get(variant) or LINEAR[variant])[index])
+    assert m.variant == variant, m.reason
+    g = torch.Generator().manual_seed(100 + index)
+
+    def close(got, want, atol, rtol=1e-2):
+        err = (got.float().cpu() - want.float()).abs()
+        assert (err <= atol + rtol * want.float().abs()).all(), f"max abs err {err.max():.4g}"
+
+    if variant in LINEAR:
+        mod = modules.get(variant, "linear", **m.kwargs)
+        if variant == "lora":
+            M, N, P, R = 16, 256, 128, 32
+            cpu = dict(X=ref.randn_half((M, N), g, 0, 0.5), W=ref.randn_half((N, P), g, 0, 0.1), A=ref.randn_half((N, R), g, 0, 0.1),
+                       B=ref.randn_half((R, P), g, 0, 0.1))
+            want = ref.lora(cpu["X"], cpu["W"], cpu["A"], cpu["B"])
+        else:
+            M, K, N = 16, 256, 192
+            cpu = dict(X=ref.randn_half((M, K), g, 0, 0.5), W1=ref.randn_half((K, N), g, 0, 0.1), W2=ref.randn_half((K, N), g, 0, 0.1))
+            want = ref.gated_mlp(cpu["X"], cpu["W1"], cpu["W2"], m.kwargs["gate"])
+        t = {k: v.cuda() for k, v in cpu.items()}
+        t["O"] = torch.zeros(tuple(want.shape), dtype=torch.float16, device="cuda")
+        mod.forward(*[t[p] for p in mod.TENSOR_PARAMS])
+        torch.cuda.synchronize()
+        close(t["O"], want, 2e-2)
+        return
+    M, N, D, P = 16, 512, 64, 40
+    H = N // D
+    rnd = lambda *sh: ref.reference_recipe(sh, g) * 20
+    cpu = dict(X=rnd(M, N), WQ=rnd(N, N), WK=rnd(N, N), WV=rnd(N, N), K_cache=rnd(H, P + M, D), V_cache=rnd(H, P + M, D))
+    if variant == "prenorm":       # |X_norm| is about 1 whatever X's amplitude: keep the unscaled scores moderate
+        for w in ("WQ", "WK", "WV"):
+            cpu[w] = cpu[w] * 0.1
+    cpu = {k: v.half() for k, v in cpu.items()}
+    cpu["noise"] = torch.randn(H, M, P + M, generator=g).half()
+    mod = modules.get(variant, "decode", head_dim=D, **m.kwargs)
+    t = {k: v.cuda() for k, v in cpu.items()}
+    t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    for c in ("C_out", "C_out1", "C_out2"):
+        t[c] = torch.zeros(H, P + M, device="cuda")
+    mod.forward(*[t[p] for p in mod.TENSOR_PARAMS])
+    torch.cuda.synchronize()
+    args = (cpu["X"], cpu["WQ"], cpu["WK"], cpu["WV"], cpu["K_cache"], cpu["V_cache"])
+    if variant in ("vanilla", "prenorm"):
+        want = ref.decode_append_vanilla(*args, P, D, prenorm=variant == "prenorm")
+    elif variant == "qknorm":
+        want = ref.decode_append_qknorm(*args, P, D)
+    elif variant == "keyformer":
+        want, pw = ref.decode_append_keyformer(*args, cpu["noise"], P, D, tau=m.kwargs["tau"])
+        close(t["C_out"], pw.sum(1), 1e-5, 5e-3)
+    else:
+        want, s1, s2 = ref.decode_append_roco(*args, P, D)
+        close(t["C_out1"], s1, 1e-5, 5e-3); close(t["C_out2"], s2, 1e-6, 5e-3)
+    close(t["O2"], ref.flatten_token_major(want), 2e-3 if variant != "prenorm" else 2e-2)
 
 
 def test_printing_round_trips_on_random_trees():

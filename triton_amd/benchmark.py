@@ -114,7 +114,7 @@ def append_record(path: str, record: dict) -> None:
 
 
 def candidates_from_ir(path: str, start: int = 0, num: Optional[int] = 10) -> List[tuple]:
-    """(ir_id, expression, variant or None, reason) for the candidates of an IR file with id >= start, at most `num`
+    """(ir_id, expression, variant or None, reason[, constructor arguments read off the IR]) for the candidates of an IR file with id >= start, at most `num`
     of them (the reference's --start / --num / --end, vanilla_llama_benchmark.py:749-753); each is recognised by its
     dataflow instead of being compiled."""
     from . import ir
@@ -123,7 +123,7 @@ def candidates_from_ir(path: str, start: int = 0, num: Optional[int] = 10) -> Li
         if ir_id < start or (num is not None and len(out) >= num):
             continue
         m = ir.recognise(expr)
-        out.append((ir_id, expr, m.variant, m.reason))
+        out.append((ir_id, expr, m.variant, m.reason, m.kwargs))
     return out
 
 
@@ -139,12 +139,13 @@ def run(variant: str, configs: List[Dict[str, int]], output: str, warmup_runs: i
         candidates = [(f"trinity_hip/{variant}", f"hand-written gfx950 module ({variant}, {form} form)", variant, "")]
     records = []
     for cfg in configs:
-        for ir_id, expr, var, reason in candidates:
+        for ir_id, expr, var, reason, *rest in candidates:
+            consts = rest[0] if rest else {}
             rec = {"ir_id": ir_id, "ir_expression": expr, "execution_time_ms": float("inf"), "tensor_config": dict(cfg), "error": None}
             try:
                 if var is None:         # the reference records a candidate it cannot compile and carries on (:206-210)
                     raise ValueError(f"unsupported IR: {reason}")
-                module = modules.get(var, "linear") if var in LINEAR_VARIANTS else modules.get(var, "decode", head_dim=cfg["D"])
+                module = modules.get(var, "linear", **consts) if var in LINEAR_VARIANTS else modules.get(var, "decode", head_dim=cfg["D"], **consts)
                 tensors = make_tensors(cfg, module.TENSOR_PARAMS)
                 rec["execution_time_ms"] = time_module(module, tensors, warmup_runs, benchmark_runs)
             except Exception as e:      # ... and one that fails at run time (:329-332)

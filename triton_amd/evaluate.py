@@ -33,14 +33,18 @@ def constants(model: str) -> Dict[str, int]:
 
 def seeded_tensors(cfg: Dict[str, int], names, device: str = "cuda"):
     """The test inputs of convert_eval_rms.py:169-214: seed 42, `randn.clamp(-1, 1) * 0.01` for X, the weights and the
-    caches, plain `randn` noise, zero outputs; drawn on the device in the reference's order so that a tensor's values
-    do not depend on which variant is evaluated."""
+    caches, plain `randn` noise, zero outputs; drawn on the device in the reference's order -- including the `X2 =
+    randn(M)` it draws between X and WQ (:175-176) -- so that every tensor holds the reference's seed-42 values whichever
+    variant is evaluated."""
     import torch
     torch.manual_seed(42)
     torch.cuda.manual_seed(42)
     shp = tensor_shapes(cfg)
     drawn = {}
-    for n in ("X", "WQ", "WK", "WV", "K_cache", "V_cache"):
+    for n in ("X", "X2", "WQ", "WK", "WV", "K_cache", "V_cache"):
+        if n == "X2":
+            torch.randn(cfg["M"], device=device, dtype=torch.float16)       # drawn and not used, as in the reference
+            continue
         drawn[n] = torch.randn(shp[n], device=device, dtype=torch.float16).clamp(-1, 1) * 0.01
     drawn["noise"] = torch.randn(shp["noise"], device=device, dtype=torch.float16)
     out = {}
@@ -54,7 +58,7 @@ def seeded_tensors(cfg: Dict[str, int], names, device: str = "cuda"):
     return out
 
 
-def eager_baseline(variant: str, t, cfg: Dict[str, int]):
+def eager_baseline(variant: str, t, cfg: Dict[str, int], tau: float = 1.5):
     """The variant in eager PyTorch, fp16 on the GPU, following ref_rms.py (:45-83 Vanila, :101-127 PreNorm,
     :147-179 KeyFormer, :197-231 QKNorm, :249-280 RoCo) with the token-major output of convert_eval_rms.py:160.
     Returns a closure that leaves the caches as it found them (it works on clones) and returns the outputs."""
@@ -82,7 +86,7 @@ def eager_baseline(variant: str, t, cfg: Dict[str, int]):
         w = F.softmax(s, dim=-1)
         o2 = (w @ Vc).permute(1, 0, 2).reshape(M, H * D)
         if variant == "keyformer":
-            return o2, F.softmax((s + t["noise"]) / 1.5, dim=-1).sum(1)
+            return o2, F.softmax((s + t["noise"]) / tau, dim=-1).sum(1)
         if variant == "roco":          # (squares of probabilities near 1/1040 are fp16 subnormals: summed in fp32)
             return o2, w.float().sum(1), w.float().pow(2).sum(1)
         return (o2,)
@@ -118,7 +122,7 @@ def test(variant: str, cfg: Dict[str, int], module, runs: int = 100) -> dict:
     if not torch.cuda.is_available():
         raise SystemExit("Error: no GPU available; the hand-written kernels have no CPU path")
     t = seeded_tensors(cfg, list(module.TENSOR_PARAMS) + (["noise"] if variant == "keyformer" else []))
-    base = eager_baseline(variant, t, cfg)              # clones the caches before the module appends to them
+    base = eager_baseline(variant, t, cfg, getattr(module, "tau", 1.5))      # clones the caches before the module appends to them
     print("=" * 50)
     print("Starting kernel execution...")
     ms = time_module(module, t, 10, runs)
@@ -174,11 +178,14 @@ def main(argv=None) -> int:
             print(f"Error: {a.case} is not a {a.t} candidate: " + (f"recognised as {m.variant}" if m else m.reason))
             return 2
         print(f"{a.case}: {m.variant} ({m.reason})")
+        consts = m.kwargs
+    else:
+        consts = {}
     if a.o in (0, 2):
         convert(a.t, cfg)
     if a.o in (1, 2):
         from . import modules
-        result = test(a.t, cfg, modules.get(a.t, "decode", head_dim=cfg["D"]))
+        result = test(a.t, cfg, modules.get(a.t, "decode", head_dim=cfg["D"], **consts))
         if a.json:
             with open(a.json, "w") as f:
                 json.dump(result, f, indent=2)

@@ -120,12 +120,17 @@ def read_ir_file(path: str) -> List[Tuple[int, str]]:
 class Val:
     srcs: FrozenSet[str] = frozenset()
     ops: FrozenSet[str] = frozenset()
+    raw: FrozenSet[str] = frozenset()     # the sources that reach the value as a linear factor or term: through
+                                          # sums, products, matrix products and numerators only
 
     def __or__(self, o: "Val") -> "Val":
-        return Val(self.srcs | o.srcs, self.ops | o.ops)
+        return Val(self.srcs | o.srcs, self.ops | o.ops, self.raw | o.raw)
 
     def via(self, op: str) -> "Val":
-        return Val(self.srcs, self.ops | {op})
+        return Val(self.srcs, self.ops | {op}, self.raw if op in _LINEAR_OPS else frozenset())
+
+
+_LINEAR_OPS = ("add", "sub", "mul", "div", "matmul", "rsum")
 
 
 _OPNAME = {"+": "add", "-": "sub", "x": "mul", "/": "div", "*": "matmul", "exp": "exp", "sqr": "sqr", "sqrt": "sqrt",
@@ -139,10 +144,11 @@ class Dataflow:
     stored: Dict[str, Val] = field(default_factory=dict)     # every name that is stored to -> what reaches it
     squares: List[Val] = field(default_factory=list)         # operand of every squaring
     ops: set = field(default_factory=set)
+    noise_divisors: set = field(default_factory=set)         # right operand of every division of a noise-carrying sum
 
     def value_of(self, name: str, kind: str) -> Val:
         v = self.stored.get(name, Val())
-        return v | Val(frozenset({name})) if kind == "input" else v
+        return v | Val(frozenset({name}), frozenset(), frozenset({name})) if kind == "input" else v
 
 
 def _names(n: Node) -> List[str]:
@@ -181,6 +187,10 @@ def analyse(tree: Union[Node, Atom]) -> Dataflow:
             if n.op == "sqr" or (n.op == "x" and n.args[0] == n.args[1]):
                 sq_out.append(vals[0])
                 return vals[0].via("sqr")
+            if n.op == "/":
+                if "noise" in vals[0].srcs and "exp" not in vals[0].ops:
+                    df.noise_divisors.add(n.args[1] if not isinstance(n.args[1], Node) else str(n.args[1]))
+                vals[1] = Val(vals[1].srcs, vals[1].ops)          # a denominator is not a linear factor
             v = Val()
             for x in vals:
                 v = v | x
@@ -220,9 +230,15 @@ def analyse(tree: Union[Node, Atom]) -> Dataflow:
 class Match:
     variant: Optional[str]          # one of modules' variants, or None
     reason: str                     # why, or why not
+    params: Tuple[Tuple[str, object], ...] = ()     # constructor arguments read off the candidate (KeyFormer's tau,
+                                                    # the gated MLP's gate), as sorted (name, value) pairs
 
     def __bool__(self) -> bool:
         return self.variant is not None
+
+    @property
+    def kwargs(self) -> Dict[str, object]:
+        return dict(self.params)
 
 
 ATTENTION_INPUTS = frozenset({"X", "WQ", "WK", "WV", "K_cache", "V_cache"})
@@ -245,7 +261,11 @@ def _recognise_linear(df: Dataflow) -> Optional[Match]:
             return Match(None, "gated-MLP inputs, but O does not depend on all of X, W1, W2")
         if not {"matmul", "mul"} <= o.ops or not ({"sigmoid"} <= o.ops or {"exp", "div"} <= o.ops):
             return Match(None, f"gated-MLP inputs, but O is not a gated product (operators {sorted(o.ops)})")
-        return Match("gmlp", "the product with W1, through a sigmoid gate, multiplies the product with W2")
+        if "W2" not in o.raw:
+            return Match(None, "gated-MLP inputs, but the product with W2 does not reach O as a factor")
+        # sigmoid(X W1) * (X W2), or SiLU: (X W1) * sigmoid(X W1) * (X W2) -- there the W1 product is also a factor
+        gate = "silu" if "W1" in o.raw else "sigmoid"
+        return Match("gmlp", f"the product with W1, through a {gate} gate, multiplies the product with W2", (("gate", gate),))
     return None
 
 
@@ -298,7 +318,19 @@ def recognise(ir: Union[str, Node]) -> Match:
     if finals == {"O2", "C_out"} and uses_noise and not kinds:
         c = df.stored["C_out"]
         if "noise" in c.srcs and "exp" in c.ops and "noise" not in o2.srcs:
-            return Match("keyformer", "noise reaches C_out through an exponential, O2 is plain attention")
+            # the temperature: what the noise-carrying scores are divided by before the exponential (none: 1)
+            if len(df.noise_divisors) > 1:
+                return Match(None, f"the perturbed scores are divided by more than one thing: {sorted(map(str, df.noise_divisors))}")
+            tau = 1.0
+            for dv in df.noise_divisors:
+                try:
+                    tau = float(dv)
+                except (TypeError, ValueError):
+                    return Match(None, f"the temperature {dv} of the perturbed scores is not a number")
+            if not tau > 0:
+                return Match(None, f"the temperature {tau} of the perturbed scores is not positive")
+            return Match("keyformer", f"noise reaches C_out through an exponential (temperature {tau:g}), O2 is plain attention",
+                         (("tau", tau),))
         return Match(None, "C_out is not a perturbed-softmax column sum")
     if uses_noise:
         return Match(None, "reads noise without the KeyFormer outputs")
