@@ -22,7 +22,6 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
     "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    *os.environ.get("TRN_HIPCC_FLAGS", "").split(),      # extra flags for experiments, e.g. -DTRN_FORCE_NW=8
 ]
 
 

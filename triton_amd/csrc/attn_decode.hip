@@ -12,12 +12,6 @@
 #include "attn.h"
 #include <mutex>
 
-// Memory order of the arrival increment.  Release/acquire at device scope makes the hand-over of the shares hold by
-// the memory model alone (the other threads' stores are ordered before it by the workgroup barrier); it costs one L2
-// write-back and one invalidate per WORKGROUP, about 1.5 us per launch.
-#ifndef TRN_ARRIVAL_ORDER
-#define TRN_ARRIVAL_ORDER __ATOMIC_ACQ_REL
-#endif
 typedef unsigned long long ulong2_t __attribute__((ext_vector_type(2)));
 
 namespace trn {
@@ -304,7 +298,10 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         if (dg == 0) publish(mine + 32 * D + 4 * q, float4_t{mstar, L, ms2, L2});
         __syncthreads();                                   // every wave's stores have been acknowledged
         __shared__ unsigned arrival;
-        if (tid == 0) arrival = __hip_atomic_fetch_add(&counters[bh], 1u, TRN_ARRIVAL_ORDER, __HIP_MEMORY_SCOPE_AGENT);
+        // (release/acquire at device scope makes the hand-over of the shares hold by the memory model alone -- the other
+        // threads' stores are ordered before it by the workgroup barrier; it costs one L2 write-back and one invalidate
+        // per WORKGROUP, about 1.5 us per launch)
+        if (tid == 0) arrival = __hip_atomic_fetch_add(&counters[bh], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();
         if (arrival != (unsigned)(a.n_split - 1)) return;
         const float* head_parts = parts + (int64_t)bh * a.n_split * PART;

@@ -221,10 +221,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
         m = mnew;
     };
 
-#ifndef TRN_OPERAND_WINDOW
-#define TRN_OPERAND_WINDOW 2
-#endif
-    constexpr int NQ = TRN_OPERAND_WINDOW < NS ? TRN_OPERAND_WINDOW : NS / 2;   // operand look-ahead in MFMA slots
+    constexpr int NQ = 2;   // operand look-ahead in MFMA slots (deeper windows measured the same)
     half8_t ka[NQ];    // K operands of the next block's S^T: a rolling window NQ MFMA slots ahead of use
     half8_t va[NQ];    // V^T operands of this block's P V: likewise
 

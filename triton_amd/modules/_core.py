@@ -35,7 +35,13 @@ from .. import ops
 
 
 class FusedModule:
-    """Base: the three-attribute protocol plus a shape-keyed workspace cache."""
+    """Base: the three-attribute protocol plus a shape-keyed workspace cache.
+
+    A module instance is for one stream at a time: its workspaces (projected queries, row normalisers, the split-key
+    counters and partial results of the decode attention) are shared by every `forward` of the instance, so two
+    forwards of the same instance that overlap on different streams race.  Give concurrent streams an instance each.
+    The cache only grows (a captured graph keeps raw pointers into it); `release()` empties it once no captured
+    graph of this instance will be replayed again."""
 
     TENSOR_PARAMS: List[str] = []
     BLOCK_PARAMS: List[str] = []
@@ -54,6 +60,10 @@ class FusedModule:
             t = torch.empty(shape, dtype=dtype, device=device)
             self._ws[key] = t
         return t
+
+    def release(self) -> None:
+        """Drop every cached workspace.  Graphs captured from this instance must not be replayed afterwards."""
+        self._ws.clear()
 
     def _split(self, args, kwargs):
         n = len(self.TENSOR_PARAMS)
