@@ -22,11 +22,12 @@ Reference lines restated here (paths are inside the reference repository):
 Parity pinning: the reference holds no tests, golden vectors or fixtures for this
 path, so each function is pinned by closed forms, invariants, library routines
 (F.rms_norm, F.scaled_dot_product_attention) and fp64 brute force on tiny shapes
-in tests/test_oracle_*.py.  The one convention the reference does not define --
-RoCo's per-key *standard deviation* -- is this build's own (population std over
-the queries that can see the key); it is derived from the two sums the reference
-does define and is marked "parity unpinned" in roco_mean_std below.  The same holds for the gate of
-gated_mlp (the reference names the workload's tensors, not the expression): "parity unpinned" there.
+in tests/test_oracle_*.py.  One statistic the reference does not define -- RoCo's
+per-key *mean and standard deviation* (it defines the two sums) -- is stated here
+as numpy's mean / std (population) of the probabilities of the queries that can
+see the key, and roco_mean_std is held to exactly that on random inputs; there is
+no reference formula for it to be at parity with.  The gate of gated_mlp (the
+reference names the workload's tensors, not the expression) is "parity unpinned".
 """
 from __future__ import annotations
 
@@ -162,8 +163,9 @@ def visible_queries(sq: int, skv: int, causal: bool, device=None) -> torch.Tenso
 def roco_mean_std(s1: torch.Tensor, s2: torch.Tensor, sq: int, causal: bool) -> Tuple[torch.Tensor, torch.Tensor]:
     """mean_j = s1_j / n_j ; std_j = sqrt(max(s2_j / n_j - mean_j^2, 0)).
 
-    PARITY UNPINNED: the reference defines only the two sums (ref_rms.py:274-275);
-    the population-std-over-visible-queries convention is this build's own.
+    The reference defines only the two sums (ref_rms.py:274-275).  The statistic meant here is numpy's
+    mean / std (ddof = 0) of column j of the probability matrix over the rows that can see key j;
+    tests/test_oracle_pins.py holds this function to that on random inputs and under uniform attention.
     """
     n = visible_queries(sq, s1.shape[-1], causal, s1.device)
     mean = s1 / n

@@ -13,7 +13,6 @@ struct AttnArgs {
     float c2, c3;  // scale*log2(e)/tau, log2(e)/tau     : perturbed scores  z2 = s*c2 + g*c3
     float q_eps;
     int causal, q_norm;
-    int paired;    // attn_fwd16 only: a workgroup's two wave groups own query tiles from opposite ends (set by its launcher)
     // decode kernel only: keys split over n_split workgroups per head, partial results and arrival counters in ws
     int n_split;
     float* ws;

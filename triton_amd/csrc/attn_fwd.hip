@@ -510,7 +510,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
-    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs; a.paired = 0;
+    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
     if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)

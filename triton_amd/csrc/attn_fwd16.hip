@@ -57,8 +57,9 @@ template <int D> __device__ __forceinline__ int swz16(int r) {
 
 struct Scores16 { float4_t s[2][2]; };      // [key half][query block]
 
-template <int D, int NW>
+template <int D, int NW, bool PAIRED>
 __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(const AttnArgs a) {
+    static_assert(!PAIRED || NW == 8, "paired query tiles are two groups of four waves");
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int BN = 64;       // keys per LDS stage (two 32-key blocks)
     constexpr int NS = D / 8;    // MFMA slots per phase: 2 key halves x 2 query blocks x D/32 steps of S^T; D/16 x 2 of P V
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     // early waves stop at their own last visible tile as they do in plain mode.
     int q0, q_last, wq0;
     bool idle = false;
-    if (NW == 8 && a.paired) {
+    if constexpr (PAIRED) {
         const int lt = (int)(blockIdx.x / BH), ht = a.n_qtiles - 1 - lt;     // n_qtiles counts 128-query tiles here
         q0 = ht * 128; q_last = q0 + 127;
         idle = wave >= 4 && lt == ht;                                       // odd tile count: the middle one is alone
@@ -414,19 +415,18 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
 #endif
 }
 
-template <int D, int NW>
+template <int D, int NW, bool PAIRED = false>
 static hipError_t launch16(AttnArgs a, hipStream_t s) {
     int64_t grid;
-    if (NW == 8 && a.paired) {
+    if (PAIRED) {
         a.n_qtiles = (a.Sq + 127) / 128;
         grid = (int64_t)((a.n_qtiles + 1) / 2) * a.B * a.Hq;
     } else {
-        a.paired = 0;
         a.n_qtiles = (a.Sq + 32 * NW - 1) / (32 * NW);
         grid = (int64_t)a.n_qtiles * a.B * a.Hq;
     }
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
-    hipLaunchKernelGGL((attn_fwd16_kernel<D, NW>), dim3((unsigned)grid), dim3(NW * 64), 0, s, a);
+    hipLaunchKernelGGL((attn_fwd16_kernel<D, NW, PAIRED>), dim3((unsigned)grid), dim3(NW * 64), 0, s, a);
     return hipGetLastError();
 }
 
@@ -447,17 +447,17 @@ Attn16Shape attn_fwd16_shape(int batch, int n_q_heads, int seq_q, int head_dim, 
 }
 
 hipError_t launch_attn_fwd16(const AttnArgs& a, int head_dim, Attn16Shape shape, hipStream_t s) {
-    AttnArgs b = a;
-    b.paired = shape == Attn16Shape::Paired ? 1 : 0;
-    const bool wide = shape != Attn16Shape::Narrow;
-    if (head_dim == 128) return wide ? launch16<128, 8>(b, s) : launch16<128, 4>(b, s);
-    return wide ? launch16<64, 8>(b, s) : launch16<64, 4>(b, s);
+    if (shape == Attn16Shape::Paired) return head_dim == 128 ? launch16<128, 8, true>(a, s) : launch16<64, 8, true>(a, s);
+    const bool wide = shape == Attn16Shape::Wide;
+    if (head_dim == 128) return wide ? launch16<128, 8>(a, s) : launch16<128, 4>(a, s);
+    return wide ? launch16<64, 8>(a, s) : launch16<64, 4>(a, s);
 }
 
 const char* attn_fwd16_kernel_name(int head_dim, Attn16Shape shape) {
-    const bool wide = shape != Attn16Shape::Narrow;
-    if (head_dim == 128) return wide ? "trn::attn_fwd16_kernel<128, 8>" : "trn::attn_fwd16_kernel<128, 4>";
-    return wide ? "trn::attn_fwd16_kernel<64, 8>" : "trn::attn_fwd16_kernel<64, 4>";
+    if (shape == Attn16Shape::Paired) return head_dim == 128 ? "trn::attn_fwd16_kernel<128, 8, true>" : "trn::attn_fwd16_kernel<64, 8, true>";
+    const bool wide = shape == Attn16Shape::Wide;
+    if (head_dim == 128) return wide ? "trn::attn_fwd16_kernel<128, 8, false>" : "trn::attn_fwd16_kernel<128, 4, false>";
+    return wide ? "trn::attn_fwd16_kernel<64, 8, false>" : "trn::attn_fwd16_kernel<64, 4, false>";
 }
 
 }  // namespace trn
