@@ -30,6 +30,7 @@ int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const voi
 
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream);
+const char* attn_decode_kernel_name(int batch, int n_q_heads, int seq_kv, int head_dim, bool noise);
 // Bytes of workspace with which launch_attn_decode splits the keys of this problem over several workgroups (0: it would not).
 int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq_kv, int head_dim);
 

@@ -18,23 +18,44 @@ namespace trn {
 
 constexpr int DNW = 8;    // waves per workgroup
 
-template <int D, bool NOISE>
+// XOR swizzle of the 16-byte chunk index of a V row as wide as this workgroup's share of the head dimension
+template <int DV> __device__ __forceinline__ int swzv(int r) {
+    if constexpr (DV == 32) return (r >> 1) & 3;          // 4 chunks per 64-byte row
+    else return swz<DV>(r);
+}
+
+// DS: the head dimension of V and O is shared out over DS workgroups per head (each computes all the scores, from
+// all of K, but streams only its DV = D / DS columns of V and writes those columns of O).  One CU pulls 40 - 55 GB/s
+// whatever its waves ask for, and with one workgroup per head that rate is what the kernel's time is made of; more
+// workgroups per head without anything to hand over between them means fewer bytes through each CU.
+template <int D, int DS, bool NOISE>
 __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
-    constexpr int NS = D / 16;    // k-steps of S^T = K Q^T; also (2 key halves) x (D/32) MFMAs of P V
-    constexpr int NDB = D / 32;
-    constexpr int CPR = D / 8;    // 16-byte chunks per row
+    constexpr int DV = D / DS;    // columns of V / O this workgroup owns
+    constexpr int NS = D / 16;    // k-steps of S^T = K Q^T
+    constexpr int NSV = DV / 16;  // (2 key halves) x (DV/32) MFMAs of P V
+    constexpr int NDB = DV / 32;
+    constexpr int CPR = DV / 8;   // 16-byte chunks per V row share
     constexpr int RPI = 64 / CPR; // rows per wave-wide 1 KB load
     constexpr int NI = 32 / RPI;  // such loads per 32-key V block
     // two V stages (each holds the eight waves' private parts), as two arrays: LDS reads are ordered after
     // outstanding global->LDS loads that may alias them, and only distinct variables are provably disjoint
-    __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * D];
-    __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * D];
+    __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * DV];
+    __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * DV];
     __shared__ float st_m[DNW][32], st_l[DNW][32], st_m2[DNW][32], st_l2[DNW][32];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int j = blockIdx.x / a.n_split, split = blockIdx.x % a.n_split;
+    // workgroup id -> (batch x head j, key share, column share).  The column shares of a head read the same K: their
+    // ids are 8 apart, so that they sit on one XCD (ids are dealt to the 8 XCDs in turn) and share its L2.
+    int j, split, dsl;
+    if constexpr (DS > 1) {
+        const int grp = blockIdx.x / (8 * DS), rem = blockIdx.x % (8 * DS);
+        j = grp * 8 + rem % 8; dsl = rem / 8; split = 0;
+        if (j >= a.B * a.Hq) return;                    // the last group of eight heads may be short
+    } else {
+        j = blockIdx.x / a.n_split; split = blockIdx.x % a.n_split; dsl = 0;
+    }
     const int G = a.Hq / a.Hkv, nkv = a.B * a.Hkv;
     const int kvslot = j % nkv, g = j / nkv;
     const int b = kvslot / a.Hkv, kvh = kvslot % a.Hkv, head = kvh * G + g;
@@ -66,12 +87,12 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
     for (int n = 0; n < NI; ++n) {
         const int r = n * RPI + lane / CPR;
-        vvo[n] = (int)(r * a.vs * 2) + (((lane % CPR) ^ swz<D>(r)) << 4);
+        vvo[n] = (int)(r * a.vs * 2) + dsl * DV * 2 + (((lane % CPR) ^ swzv<DV>(r)) << 4);
     }
     const int vblk_bytes = (int)(32 * a.vs * 2);
 #define TRN_FETCH_V(blk_, dst_)                                                                                  \
     _Pragma("unroll") for (int n_ = 0; n_ < NI; ++n_) __builtin_amdgcn_raw_ptr_buffer_load_lds(                  \
-        vrs, (__attribute__((address_space(3))) void*)(&dst_[wave * 32 * D + n_ * RPI * D]), 16, vvo[n_],        \
+        vrs, (__attribute__((address_space(3))) void*)(&dst_[wave * 32 * DV + n_ * RPI * DV]), 16, vvo[n_],      \
         (blk_) * vblk_bytes, 0, 0)
     // V^T operand through the transposing read (as in the prefill kernel): rows 4h + (lane%16)/4 [+8] of a 16-key half
     int voff_lo[NDB], voff_hi[NDB];
@@ -80,8 +101,8 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         const int lc = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1), sub = (lane & 1) * 4;
 #pragma unroll
         for (int db = 0; db < NDB; ++db) {
-            voff_lo[db] = wave * 32 * D + rl * D + (((db * 4 + lc) ^ swz<D>(rl)) << 3) + sub;
-            voff_hi[db] = wave * 32 * D + rh * D + (((db * 4 + lc) ^ swz<D>(rh)) << 3) + sub;
+            voff_lo[db] = wave * 32 * DV + rl * DV + (((db * 4 + lc) ^ swzv<DV>(rl)) << 3) + sub;
+            voff_hi[db] = wave * 32 * DV + rh * DV + (((db * 4 + lc) ^ swzv<DV>(rh)) << 3) + sub;
         }
     }
 
@@ -174,8 +195,8 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         constexpr int kBehind = NS + NI + (NOISE ? 4 : 0);
         __builtin_amdgcn_s_waitcnt(0x0f70 | (kBehind & 15) | ((kBehind >> 4) << 14));
 #pragma unroll
-        for (int i = 0; i < NS; ++i) {
-            const half_t* vp = Vc + 16 * (i / NDB) * D;
+        for (int i = 0; i < NSV; ++i) {
+            const half_t* vp = Vc + 16 * (i / NDB) * DV;
             const half4_t lo = lds_read_tr16(vp + voff_lo[i % NDB]);
             const half4_t hi = lds_read_tr16(vp + voff_hi[i % NDB]);
             const half8_t va = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
@@ -221,7 +242,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #undef TRN_FETCH_V
 
     // ---- merge the eight waves' (m, l, O^T) through LDS.  Partial O^T as float4 quads [d/4][query]: the first half
-    // of head_dim in this wave's part of Vs0, the second half in its part of Vs1 (each exactly 32 * D/2 floats).
+    // of the columns in this wave's part of Vs0, the second half in its part of Vs1 (each exactly 32 * DV/2 floats).
     l = half_sum(l);
     __builtin_amdgcn_s_waitcnt(0x0f70);                 // the look-ahead requests past the end have landed too
     if (h == 0) { st_m[wave][c] = m; st_l[wave][c] = l; }
@@ -231,15 +252,17 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     }
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
-        float4_t* part = reinterpret_cast<float4_t*>((db < NDB / 2 ? Vs0 : Vs1) + wave * 32 * D);
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            part[((db % (NDB / 2)) * 8 + 2 * r4 + h) * 32 + c] =
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int quad = db * 8 + 2 * r4 + h;             // columns 4 quad .. +3 of this workgroup's share
+            float4_t* part = reinterpret_cast<float4_t*>((quad < DV / 8 ? Vs0 : Vs1) + wave * 32 * DV);
+            part[(quad % (DV / 8)) * 32 + c] =
                 float4_t{oacc[db][r4 * 4], oacc[db][r4 * 4 + 1], oacc[db][r4 * 4 + 2], oacc[db][r4 * 4 + 3]};
+        }
     }
     __syncthreads();
-    const int q = tid & 31, dg = tid >> 5;                // 16 groups of threads share out the D/4 quads of a query
-    constexpr int NQD = (D / 4) / 16;                     // quads per thread
+    const int q = tid & 31, dg = tid >> 5;                // 16 groups of threads share out the DV/4 quads of a query
+    constexpr int NQD = (DV / 4 + 15) / 16;               // quads per thread (with 8 quads, half the groups have none)
     float mstar = st_m[0][q];
 #pragma unroll
     for (int w = 1; w < DNW; ++w) mstar = fmaxf(mstar, st_m[w][q]);
@@ -254,12 +277,12 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         }
 #pragma unroll
         for (int qi = 0; qi < NQD; ++qi) {
-            const int quad = dg + 16 * qi;                // d = 4*quad .. +3
-            const half_t* base = quad < D / 8 ? Vs0 : Vs1;
-            const int ql = quad % (D / 8);
+            const int quad = min(dg + 16 * qi, DV / 4 - 1);   // d = 4*quad .. +3 (a group without a quad re-reads the last)
+            const half_t* base = quad < DV / 8 ? Vs0 : Vs1;
+            const int ql = quad % (DV / 8);
             acc[qi] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int w = 0; w < DNW; ++w) acc[qi] += reinterpret_cast<const float4_t*>(base + w * 32 * D)[ql * 32 + q] * wgt[w];
+            for (int w = 0; w < DNW; ++w) acc[qi] += reinterpret_cast<const float4_t*>(base + w * 32 * DV)[ql * 32 + q] * wgt[w];
         }
     }
     float ms2 = -INFINITY, L2 = 0.f;
@@ -270,7 +293,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         for (int w = 0; w < DNW; ++w) L2 += ms2 == -INFINITY ? 0.f : st_l2[w][q] * fast_exp2(st_m2[w][q] - ms2);
     }
     const int bh = b * a.Hq + head;
-    if (a.n_split > 1) {
+    if (DS == 1 && a.n_split > 1) {
         // ---- keys split over workgroups: publish (m, l, unnormalised O) of this share; the workgroup that arrives
         // last at the head's counter merges all shares.  Workspace: [arrival counters, 256-byte aligned][bh][split]
         // {O as quads [D/4][32 queries][4], (m, l, m2, l2) [32]} floats.  The shares travel as device-scope atomic stores and loads, which
@@ -344,24 +367,26 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     }
     {
         const float inv = 1.0f / L;
-        half_t* orow = a.o + b * a.ob + head * a.oh + (int64_t)q * a.os;
+        half_t* orow = a.o + b * a.ob + head * a.oh + (int64_t)q * a.os + dsl * DV;
         if (q < a.Sq) {
 #pragma unroll
             for (int qi = 0; qi < NQD; ++qi) {
                 const half4_t ov = {(half_t)(acc[qi][0] * inv), (half_t)(acc[qi][1] * inv), (half_t)(acc[qi][2] * inv), (half_t)(acc[qi][3] * inv)};
-                *reinterpret_cast<half4_t*>(orow + 4 * (dg + 16 * qi)) = ov;
+                if (dg + 16 * qi < DV / 4) *reinterpret_cast<half4_t*>(orow + 4 * (dg + 16 * qi)) = ov;
             }
         }
-        if (dg == 0 && q < a.Sq && a.lse) a.lse[(int64_t)bh * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
+        // (every column share holds the same row normalisers: the first one writes them)
+        if (dg == 0 && dsl == 0 && q < a.Sq && a.lse) a.lse[(int64_t)bh * a.Sq + q] = (mstar + fast_log2(L)) * kLn2;
         if constexpr (NOISE) {
-            if (dg == 1 && q < a.Sq) a.lse_pert[(int64_t)bh * a.Sq + q] = (ms2 + fast_log2(L2)) * kLn2;
+            if (dg == 1 && dsl == 0 && q < a.Sq) a.lse_pert[(int64_t)bh * a.Sq + q] = (ms2 + fast_log2(L2)) * kLn2;
         }
     }
     // ---- column statistics (KeyFormer key scores, RoCo sums): a second sweep over this head's keys now that the
     // row normalisers are final.  The score block is formed the other way round, S[query][key] -- the same two
     // register operands with their roles swapped -- so that a lane owns one KEY and holds 16 of the 32 queries: the
     // sum over queries is in-lane plus one exchange with lane^32, and a block's 32 sums are one 128-byte store.
-    // (Only with one workgroup per head: the launcher does not split the keys when these outputs are asked for.)
+    // (Not with the keys split over workgroups -- the statistics need the normalisers of the whole head; the column
+    // shares of a head all have them, and take every DS-th round of blocks of the sweep each.)
     if (a.col_sum || a.col_sumsq || a.probs) {
         __syncthreads();                                   // every thread has read the merge arrays
         if (dg == 0) st_l[0][q] = NOISE ? ms2 + fast_log2(L2) : mstar + fast_log2(L);     // log2 domain
@@ -386,9 +411,9 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         // L2, about 55 GB/s; requesting two blocks ahead measured the same)
         auto sweep = [&](int it, half8_t (&kc)[NS], half8_t (&kn)[NS], float (&gc)[NOISE ? 16 : 1], float (&gn)[NOISE ? 16 : 1])
                          __attribute__((always_inline)) {
-            const int blk = blk0 + wave + it * DNW, key = blk * 32 + c;
-            fetch_k(blk + DNW, kn);
-            fetch_noise_col(blk + DNW, gn);
+            const int blk = blk0 + dsl * DNW + wave + it * DNW * DS, key = blk * 32 + c;
+            fetch_k(blk + DNW * DS, kn);
+            fetch_noise_col(blk + DNW * DS, gn);
             float16_t s;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = 0.f;
@@ -413,11 +438,13 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
                 if (a.col_sumsq) a.col_sumsq[(int64_t)bh * a.Skv + key] = y;
             }
         };
-        fetch_k(blk0 + wave, ka0);
-        fetch_noise_col(blk0 + wave, gs0);
-        for (int it = 0; it < nmine; it += 2) {
+        const int first = dsl * DNW + wave;
+        const int nsweep = nblk > first ? (nblk - first + DNW * DS - 1) / (DNW * DS) : 0;
+        fetch_k(blk0 + first, ka0);
+        fetch_noise_col(blk0 + first, gs0);
+        for (int it = 0; it < nsweep; it += 2) {
             sweep(it, ka0, ka1, gs0, gs1);
-            if (it + 1 < nmine) sweep(it + 1, ka1, ka0, gs1, gs0);
+            if (it + 1 < nsweep) sweep(it + 1, ka1, ka0, gs1, gs0);
         }
     }
 #endif
@@ -445,6 +472,25 @@ int64_t attn_decode_workspace_bytes(int batch, int n_q_heads, int seq_q, int seq
     return ((n_bh + 63) / 64) * 256 + n_bh * ns * 32 * (head_dim + 4) * 4;
 }
 
+static int decode_col_shares(int64_t n_bh, int seq_kv, int head_dim) {
+    int ds = 1;
+    if (seq_kv >= 256)
+        while (ds < 4 && head_dim / (ds * 2) >= 32 && n_bh * ds * 2 <= 256) ds *= 2;
+    return ds;
+}
+
+// Name of the instantiation launched for a problem without a workspace (a measurement aid: what a kernel trace shows).
+const char* attn_decode_kernel_name(int batch, int n_q_heads, int seq_kv, int head_dim, bool noise) {
+    const int ds = decode_col_shares((int64_t)batch * n_q_heads, seq_kv, head_dim);
+    if (head_dim == 128) {
+        if (ds == 4) return noise ? "trn::attn_decode_kernel<128, 4, true>" : "trn::attn_decode_kernel<128, 4, false>";
+        if (ds == 2) return noise ? "trn::attn_decode_kernel<128, 2, true>" : "trn::attn_decode_kernel<128, 2, false>";
+        return noise ? "trn::attn_decode_kernel<128, 1, true>" : "trn::attn_decode_kernel<128, 1, false>";
+    }
+    if (ds == 2) return noise ? "trn::attn_decode_kernel<64, 2, true>" : "trn::attn_decode_kernel<64, 2, false>";
+    return noise ? "trn::attn_decode_kernel<64, 1, true>" : "trn::attn_decode_kernel<64, 1, false>";
+}
+
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
     a.n_split = 1; a.ws = nullptr;
     const int64_t need = attn_decode_workspace_bytes(a.B, a.Hq, a.Sq, a.Skv, head_dim);
@@ -452,16 +498,23 @@ hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t
         a.n_split = decode_splits(a.B, a.Hq, a.Skv, head_dim);
         a.ws = static_cast<float*>(workspace);
     }
-    const int64_t grid = (int64_t)a.B * a.Hq * a.n_split;
+    // Without a key split: share V's columns out over workgroups while that still leaves every workgroup 32 columns
+    // and the grid within one workgroup per CU (32 heads of 128: 4 shares; 71 heads of 64: 2).  Short caches are left
+    // alone: below some 8 blocks per wave-round the fixed part of a launch is all there is.
+    const int64_t n_bh = (int64_t)a.B * a.Hq;
+    const int ds = a.n_split == 1 ? decode_col_shares(n_bh, a.Skv, head_dim) : 1;
+    const int64_t grid = ds > 1 ? ((n_bh + 7) / 8) * 8 * ds : n_bh * a.n_split;
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 g((unsigned)grid), t(DNW * 64);
+#define TRN_DEC(D_, DS_, N_) hipLaunchKernelGGL((attn_decode_kernel<D_, DS_, N_>), g, t, 0, stream, a)
     if (a.noise) {
-        if (head_dim == 128) hipLaunchKernelGGL((attn_decode_kernel<128, true>), g, t, 0, stream, a);
-        else hipLaunchKernelGGL((attn_decode_kernel<64, true>), g, t, 0, stream, a);
+        if (head_dim == 128) { if (ds == 4) TRN_DEC(128, 4, true); else if (ds == 2) TRN_DEC(128, 2, true); else TRN_DEC(128, 1, true); }
+        else { if (ds == 2) TRN_DEC(64, 2, true); else TRN_DEC(64, 1, true); }
     } else {
-        if (head_dim == 128) hipLaunchKernelGGL((attn_decode_kernel<128, false>), g, t, 0, stream, a);
-        else hipLaunchKernelGGL((attn_decode_kernel<64, false>), g, t, 0, stream, a);
+        if (head_dim == 128) { if (ds == 4) TRN_DEC(128, 4, false); else if (ds == 2) TRN_DEC(128, 2, false); else TRN_DEC(128, 1, false); }
+        else { if (ds == 2) TRN_DEC(64, 2, false); else TRN_DEC(64, 1, false); }
     }
+#undef TRN_DEC
     return hipGetLastError();
 }
 

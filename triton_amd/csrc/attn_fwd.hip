@@ -427,8 +427,7 @@ extern "C" const char* trn_attn_fwd_kernel_name(const trn_attn_desc* d, int32_t 
     using namespace trn;
     if (!d || validate_attn(d, true) != TRN_OK) return "";
     const bool d128 = d->head_dim == 128;
-    if (d->seq_q <= 32) return with_noise ? (d128 ? "trn::attn_decode_kernel<128, true>" : "trn::attn_decode_kernel<64, true>")
-                                          : (d128 ? "trn::attn_decode_kernel<128, false>" : "trn::attn_decode_kernel<64, false>");
+    if (d->seq_q <= 32) return attn_decode_kernel_name(d->batch, d->n_q_heads, d->seq_kv, d->head_dim, with_noise != 0);
     if (!with_noise) return attn_fwd16_kernel_name(d->head_dim, attn_fwd16_shape(d->batch, d->n_q_heads, d->seq_q, d->head_dim, d->causal != 0));
     const bool wide = noise_kernel_wide(d);
     if (d128) return wide ? "trn::attn_fwd_kernel<128, 8, true>" : "trn::attn_fwd_kernel<128, 4, true>";
@@ -513,7 +512,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
-    if (((int64_t)d->seq_kv + 512) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 512) * d->v_stride_s * 2 > 0x7fffffffLL)
+    if (((int64_t)d->seq_kv + 2048) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 2048) * d->v_stride_s * 2 > 0x7fffffffLL)
         return TRN_E_UNSUPPORTED;
     hipStream_t s = (hipStream_t)stream;
     hipError_t e;
