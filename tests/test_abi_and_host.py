@@ -99,6 +99,32 @@ def test_validation_rejects_before_launch(lib):
     assert g(tokens=0) == 0
 
 
+def test_kernel_name_follows_the_launch_rules(lib):
+    """trn_attn_fwd_kernel_name answers from the same rules the launch uses (no device involved): the workgroup shape
+    of the 16x16x32 kernel by problem size, the kernel with score perturbation, the decode kernel with its column
+    shares."""
+    def name(with_noise=0, **kw):
+        S, Skv, D, H = kw.get("seq_q", 8), kw.get("seq_kv", kw.get("seq_q", 8)), kw.get("head_dim", 64), kw.get("n_q_heads", 4)
+        kw.setdefault("seq_kv", Skv)
+        strides = dict(q_stride_b=H * S * D, q_stride_h=S * D, q_stride_s=D, o_stride_b=H * S * D, o_stride_h=S * D, o_stride_s=D,
+                       k_stride_b=kw.get("n_kv_heads", 2) * Skv * D, k_stride_h=Skv * D, k_stride_s=D,
+                       v_stride_b=kw.get("n_kv_heads", 2) * Skv * D, v_stride_h=Skv * D, v_stride_s=D)
+        return lib.trn_attn_fwd_kernel_name(C.byref(_desc(**strides, **kw)), with_noise).decode()
+    llama = dict(n_q_heads=32, n_kv_heads=8, head_dim=128)
+    assert name(seq_q=4096, **llama) == "trn::attn_fwd16_kernel<128, 8, false>"         # two rounds of wide workgroups
+    assert name(seq_q=2048, **llama) == "trn::attn_fwd16_kernel<128, 8, true>"          # a single round: paired tiles
+    assert name(seq_q=1024, **llama) == "trn::attn_fwd16_kernel<128, 4, false>"         # pairs would cover half the chip
+    assert name(seq_q=4096, causal=0, **llama) == "trn::attn_fwd16_kernel<128, 8, false>"
+    assert name(seq_q=2048, n_q_heads=71, n_kv_heads=1, head_dim=64) == "trn::attn_fwd16_kernel<64, 4, false>"
+    assert name(1, seq_q=4096, **llama) == "trn::attn_fwd_kernel<128, 8, true>"
+    assert name(1, seq_q=512, **llama) == "trn::attn_fwd_kernel<128, 4, true>"
+    assert name(seq_q=16, seq_kv=1040, causal=0, **llama) == "trn::attn_decode_kernel<128, 4, false>"
+    assert name(1, seq_q=16, seq_kv=1040, causal=0, n_q_heads=71, n_kv_heads=71, head_dim=64) == "trn::attn_decode_kernel<64, 2, true>"
+    assert name(seq_q=16, seq_kv=100, causal=0, **llama) == "trn::attn_decode_kernel<128, 1, false>"    # short cache
+    assert name(seq_q=16, seq_kv=1040, causal=0, n_q_heads=160, n_kv_heads=8, head_dim=128) == "trn::attn_decode_kernel<128, 1, false>"
+    assert name(head_dim=32) == ""                                                                 # invalid descriptor
+
+
 def test_validation_of_the_workspace_statistics_and_linear_entry_points(lib):
     """As above: every call fails validation before anything is launched."""
     p = C.c_void_p(0x1000)

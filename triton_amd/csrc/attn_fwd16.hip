@@ -249,9 +249,12 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     // Every LDS operand feeds two consecutive MFMAs (the two query blocks); it is requested NQ operands before its
     // first use, into the register its predecessor has just vacated.  With SYNC (first block of a 64-key tile) the
     // tile hand-over sits right after the last request to the tile's own K stage.
-    auto step = [&](bool masked_next, auto sync_tag, Scores16& sc, Scores16& sn, const half_t* Vblk, const half_t* K1,
+    // MAYMASK = false: the caller knows that block B+1 needs no mask, and the test and its branch (which would sit in
+    // the middle of phase B and split the slot sequence) are not compiled in.
+    auto step = [&](bool masked_next, auto maymask_tag, auto sync_tag, Scores16& sc, Scores16& sn, const half_t* Vblk, const half_t* K1,
                     const half_t* K2, int key0_next, auto&& handover) __attribute__((always_inline)) {
         constexpr bool SYNC = decltype(sync_tag)::value;
+        constexpr bool MAYMASK = decltype(maymask_tag)::value;
         half8_t pB[2];
         auto load_v = [&](int db, int reg) __attribute__((always_inline)) {
             const half4_t lo = lds_read_tr16(Vblk + voff[db]);              // keys 4 g4 .. +3, dim 16 db + n
@@ -294,7 +297,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
                 if (db + NQ < NOP) load_v(db + NQ, db % NQ);
                 else load_k(K2, db + NQ - NOP, db % NQ);
             }
-            if (i == NS / 2) due = reduce_block(masked_next, sn, key0_next, smax);
+            if (i == NS / 2) due = reduce_block(MAYMASK && masked_next, sn, key0_next, smax);
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
@@ -335,18 +338,20 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
 
     // One 64-key tile jt.  Kc = its own K stage (block 1 still has operands to give), Kn = the next tile's
     // K stage, Vc = its V stage, Vn = the other V stage.
-    auto tile = [&](int jt, half_t* Kc, const half_t* Kn, const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
+    auto tile = [&](auto maymask_tag, int jt, half_t* Kc, const half_t* Kn, const half_t* Vc, half_t* Vn) __attribute__((always_inline)) {
         const int kv0 = jt * BN;
         auto handover = [&]() __attribute__((always_inline)) {
             __builtin_amdgcn_s_waitcnt(0x0f70);   // this wave's share of stages Kn and Vc is in LDS
             __syncthreads();                      // ... and everyone's; Kc and Vn have had their last readers
-            if (jt + 2 < ntiles) TRN_FETCH_K(jt + 2, Kc);
-            if (jt + 1 < ntiles) TRN_FETCH_V(jt + 1, Vn);
+            // (unconditional: tiles past the end of the keys read as zeros into stages nobody reads, and the
+            // hand-over stays free of branches)
+            TRN_FETCH_K(jt + 2, Kc);
+            TRN_FETCH_V(jt + 1, Vn);
         };
         auto none = [&]() __attribute__((always_inline)) {};
         // (Past the last tile a K stage holds stale rows; scores computed from them are masked away.)
-        step(needs_mask(kv0 + 32), std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
-        step(needs_mask(kv0 + 64), std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
+        step(needs_mask(kv0 + 32), maymask_tag, std::true_type{}, sA, sB, Vc, Kc + 32 * D, Kn, kv0 + 32, handover);
+        step(needs_mask(kv0 + 64), maymask_tag, std::false_type{}, sB, sA, Vc + 32 * D, Kn, Kn + 32 * D, kv0 + 64, none);
     };
     // Under a causal mask the waves of a workgroup see different numbers of tiles: a wave computes the tiles that
     // hold a key visible to one of its queries, and for the rest only keeps up the staging it shares with the
@@ -354,9 +359,20 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     int nlive = ntiles;
     if (a.causal) nlive = min(ntiles, (min(wq0 + 31, a.Sq - 1) + off) / BN + 1);
     if (idle) nlive = 0;
-    for (int jt = 0; jt < nlive; jt += 2) {
-        tile(jt, Ks0, Ks1, Vs0, Vs1);
-        if (jt + 1 < nlive) tile(jt + 1, Ks1, Ks0, Vs1, Vs0);
+    // The leading tiles whose blocks (and the first block of the tile after) lie wholly inside the keys and, under a
+    // causal mask, before this wave's first query: a loop of their own without the mask test.  needs_mask is monotone
+    // in the key index, so they are the tiles jt with 64 jt + 96 <= Skv and 64 jt + 95 <= wb; taken in pairs (the
+    // stages alternate), the rest goes through the general loop.
+    int n_plain = (a.Skv - 96 >= 0) ? (a.Skv - 96) / BN + 1 : 0;
+    if (a.causal) n_plain = min(n_plain, wb - 95 >= 0 ? (wb - 95) / BN + 1 : 0);
+    n_plain = min(n_plain, nlive) & ~1;
+    for (int jt = 0; jt < n_plain; jt += 2) {
+        tile(std::false_type{}, jt, Ks0, Ks1, Vs0, Vs1);
+        tile(std::false_type{}, jt + 1, Ks1, Ks0, Vs1, Vs0);
+    }
+    for (int jt = n_plain; jt < nlive; jt += 2) {
+        tile(std::true_type{}, jt, Ks0, Ks1, Vs0, Vs1);
+        if (jt + 1 < nlive) tile(std::true_type{}, jt + 1, Ks1, Ks0, Vs1, Vs0);
     }
     for (int jt = nlive; jt < ntiles; ++jt) {
         half_t* Kc = (jt & 1) ? Ks1 : Ks0;
@@ -375,7 +391,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     float l[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) { l[qb] = lacc[qb][0]; inv[qb] = 1.0f / l[qb]; }
-    __syncthreads();                                   // every wave is done with the K/V stages
+    __builtin_amdgcn_s_waitcnt(0x0f70);                // this wave's last refills (past the end, unread) have landed ...
+    __syncthreads();                                   // ... and everyone's; every wave is done with the K/V stages
     {
         // two passes of D/2 columns each, so that NW waves' staging regions fit in the four stage arrays
         constexpr int DP = D / 2, OP = DP + 4;         // row pitch in halfs
