@@ -161,8 +161,8 @@ int trn_attn_colstats_f16(const trn_attn_desc* desc, const void* q, const void* 
                           float* out_sum, float* out_sumsq, void* stream);
 
 /*
- * RoCo's statistics as mean and standard deviation (BASELINE workload "per-key column mean and std of the attention
- * probabilities"): out_mean[j] = (1/n_j) sum_i p_ij and out_std[j] = sqrt((1/n_j) sum_i p_ij^2 - out_mean[j]^2), the
+ * RoCo's statistics as mean and standard deviation (the per-key column mean and std of the attention
+ * probabilities): out_mean[j] = (1/n_j) sum_i p_ij and out_std[j] = sqrt((1/n_j) sum_i p_ij^2 - out_mean[j]^2), the
  * population standard deviation, over the n_j queries that can see key j (all seq_q of them without a mask;
  * seq_q - max(0, j - (seq_kv - seq_q)) under a causal mask).  The reference defines the two sums only
  * (ref_rms.py:274-275); these are formed from them in the same kernel's epilogue.  Arguments as

@@ -55,7 +55,7 @@ CASES = [
     (1, 96, 8, 600, 600, 128, True),
     (1, 96, 8, 600, 700, 128, True),
     (2, 64, 64, 500, 500, 64, True),
-    (1, 32, 8, 2048, 2048, 128, True),   # the attention of the PreNorm block (BASELINE config 3)
+    (1, 32, 8, 2048, 2048, 128, True),   # the attention of the PreNorm block (the 2048-token PreNorm workload)
 ]
 
 
