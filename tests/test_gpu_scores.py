@@ -34,7 +34,11 @@ def run_roco(q, k, v, scale, causal):
 
 CASES = [(1, 4, 2, 256, 256, 128, True), (1, 4, 2, 256, 256, 128, False), (2, 3, 1, 200, 200, 64, True),
          (1, 2, 2, 16, 1040, 128, False), (1, 2, 2, 16, 1040, 64, True), (1, 8, 2, 640, 640, 128, True),
-         (1, 1, 1, 1, 1, 64, True), (1, 2, 1, 130, 259, 128, True)]
+         (1, 1, 1, 1, 1, 64, True), (1, 2, 1, 130, 259, 128, True),
+         # longer walks of the statistics pass: several mask-free turns of its stage ring, key tiles in pairs with a
+         # middle one left over, more queries than keys without a mask, a long cached prefix under the mask
+         (1, 1, 1, 1024, 1024, 128, True), (1, 2, 1, 700, 300, 128, False), (1, 2, 2, 520, 1000, 64, True),
+         (1, 2, 1, 1100, 1100, 64, True)]
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", CASES)

@@ -391,10 +391,8 @@ __global__ __launch_bounds__(256, 2) void attn_colstats_plain_kernel(const ColAr
                     const float t = __builtin_fmaf(blk ? ac1[r] : ac0[r], a.c1, -lse2[blk]);
                     float p = fast_exp2(t);
                     if constexpr (MAYMASK) p = (8 * (r / 4) + (r % 4) <= last[blk]) ? p : 0.f;
-                    // (the running sums are updated in place, said in so many words: left to itself the compiler
-                    // rotates them through fresh registers and runs out of them)
-                    asm volatile("v_add_f32 %0, %1, %0" : "+v"(s1[r]) : "v"(p));
-                    if constexpr (SQ) asm volatile("v_fmac_f32 %0, %1, %1" : "+v"(s2[r]) : "v"(p));
+                    s1[r] += p;
+                    if constexpr (SQ) s2[r] = __builtin_fmaf(p, p, s2[r]);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
