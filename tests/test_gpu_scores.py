@@ -56,7 +56,9 @@ def test_roco_parity(B, Hq, Hkv, Sq, Skv, D, causal):
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,tau", [
     (1, 4, 2, 256, 256, 128, True, 1.0), (1, 4, 2, 200, 200, 128, True, 1.5), (1, 3, 1, 96, 96, 64, False, 1.0),
     (1, 2, 2, 16, 1040, 128, False, 1.5), (1, 2, 1, 130, 260, 64, True, 1.0),
-    (2, 4, 2, 9, 700, 128, True, 1.5), (1, 3, 1, 32, 100, 64, True, 1.0)])     # decode kernel with noise, GQA / MQA
+    (2, 4, 2, 9, 700, 128, True, 1.5), (1, 3, 1, 32, 100, 64, True, 1.0),     # decode kernel with noise, GQA / MQA
+    # longer walks of both passes: several turns of the statistics pass's stage ring, a cached prefix, both widths
+    (1, 2, 1, 600, 600, 64, True, 1.0), (1, 2, 2, 520, 1000, 128, True, 1.5), (1, 2, 1, 700, 300, 64, False, 1.0)])
 def test_keyformer_parity(B, Hq, Hkv, Sq, Skv, D, causal, tau):
     from triton_amd import ops
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=7)
