@@ -186,6 +186,21 @@ int trn_attn_fwd_stats_f16(const trn_attn_desc* desc, const void* q, const void*
                            float* out_sum, float* out_sumsq, void* stream);
 
 /*
+ * trn_attn_fwd_stats_f16 with the noise and the statistics in fp16, for the reference's decode-append problem
+ * (seq_q <= 32; TRN_E_UNSUPPORTED otherwise): its drivers allocate every tensor as fp16 -- C_out, C_out1, C_out2
+ * (vanilla_llama_benchmark.py:131-139) and the noise (convert_eval_rms.py:201) -- and this entry point takes them as
+ * they are, one launch, no widened copy of the noise and no narrowing copy of the scores.
+ *   noise       nullable fp16 [batch, n_q_heads, seq_q, seq_kv]; the strides in desc count fp16 elements; base and
+ *               pitches multiples of 8 bytes (seq_kv itself may be anything: pad the rows).
+ *   out_sum, out_sumsq   fp16 [batch, n_q_heads, seq_kv] contiguous (one may be NULL): the fp32 sums of
+ *               trn_attn_fwd_stats_f16 rounded to nearest once.
+ */
+int trn_attn_fwd_stats_half_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                                void* o, float* lse, const void* gamma_q,
+                                const void* noise, float* lse_pert,
+                                void* out_sum, void* out_sumsq, void* stream);
+
+/*
  * The decode-append form of KeyFormer as its reference class returns it (ref_rms.py:171-179): the attention output
  * and the UN-REDUCED probabilities  out_probs[b,h,i,j] = softmax_j((scale*QK^T + noise)/tau)  (plain softmax(scale*QK^T)
  * when noise is NULL), float [batch, n_q_heads, seq_q, seq_kv] contiguous, masked entries 0; optionally their sums

@@ -118,10 +118,10 @@ def test_kernel_name_follows_the_launch_rules(lib):
     assert name(seq_q=2048, n_q_heads=71, n_kv_heads=1, head_dim=64) == "trn::attn_fwd16_kernel<64, 4, false>"
     assert name(1, seq_q=4096, **llama) == "trn::attn_fwd_kernel<128, 8, true>"
     assert name(1, seq_q=512, **llama) == "trn::attn_fwd_kernel<128, 4, true>"
-    assert name(seq_q=16, seq_kv=1040, causal=0, **llama) == "trn::attn_decode_kernel<128, 4, false>"
-    assert name(1, seq_q=16, seq_kv=1040, causal=0, n_q_heads=71, n_kv_heads=71, head_dim=64) == "trn::attn_decode_kernel<64, 2, true>"
-    assert name(seq_q=16, seq_kv=100, causal=0, **llama) == "trn::attn_decode_kernel<128, 1, false>"    # short cache
-    assert name(seq_q=16, seq_kv=1040, causal=0, n_q_heads=160, n_kv_heads=8, head_dim=128) == "trn::attn_decode_kernel<128, 1, false>"
+    assert name(seq_q=16, seq_kv=1040, causal=0, **llama) == "trn::attn_decode_kernel<128, 4, 0>"
+    assert name(1, seq_q=16, seq_kv=1040, causal=0, n_q_heads=71, n_kv_heads=71, head_dim=64) == "trn::attn_decode_kernel<64, 2, 1>"
+    assert name(seq_q=16, seq_kv=100, causal=0, **llama) == "trn::attn_decode_kernel<128, 1, 0>"    # short cache
+    assert name(seq_q=16, seq_kv=1040, causal=0, n_q_heads=160, n_kv_heads=8, head_dim=128) == "trn::attn_decode_kernel<128, 1, 0>"
     assert name(head_dim=32) == ""                                                                 # invalid descriptor
 
 

@@ -262,3 +262,46 @@ def test_fused_statistics_argument_rules():
     assert e.value.status_name == "TRN_E_NULL"
     with pytest.raises(ValueError):
         ops.attention_with_stats(qd, kd, vd, o, 0.125, True, None, None)
+
+
+# ---- trn_attn_fwd_stats_half_f16: the same launch with fp16 noise and fp16 statistics (the reference's own tensors)
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,with_noise", [
+    (1, 4, 4, 16, 1040, 128, False, True), (1, 4, 2, 16, 1040, 128, True, False), (2, 6, 1, 7, 332, 64, True, True),
+    (1, 71, 1, 16, 1040, 64, False, False), (1, 3, 3, 32, 36, 128, True, True), (1, 2, 2, 1, 100, 64, False, True)])
+def test_fused_statistics_with_fp16_noise_and_outputs(B, Hq, Hkv, Sq, Skv, D, causal, with_noise):
+    """Held to the fp32 form of the same call bit for bit: the fp16 noise widened is the same noise, and an fp16 statistic
+    is the fp32 one rounded once.  (The fp32 form is held to the oracle above.)"""
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=17)
+    scale, tau = D ** -0.5, 1.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    g = torch.Generator().manual_seed(5)
+    pitch = (Skv + 3) // 4 * 4
+    n16 = torch.full((B, Hq, Sq, pitch), float("nan"), dtype=torch.float16)
+    n16[..., :Skv] = torch.randn(B, Hq, Sq, Skv, generator=g).half()
+    n16 = n16.cuda()[..., :Skv] if with_noise else None
+    n32 = None
+    if with_noise:
+        buf = torch.full((B, Hq, Sq, pitch), float("nan"), device="cuda"); buf[..., :Skv] = n16.float(); n32 = buf[..., :Skv]
+    o1 = torch.zeros_like(qd); o2 = torch.zeros_like(qd)
+    lp1 = torch.zeros(B, Hq, Sq, device="cuda"); lp2 = torch.zeros_like(lp1)
+    a1 = torch.full((B, Hq, Skv), -1.0, device="cuda"); a2 = torch.full((B, Hq, Skv), -1.0, device="cuda")
+    h1 = torch.full((B, Hq, Skv), -1.0, device="cuda", dtype=torch.float16); h2 = torch.full_like(h1, -1.0)
+    kw32 = dict(noise=n32, tau=tau, lse_pert=lp1) if with_noise else dict(lse=lp1)
+    kw16 = dict(noise=n16, tau=tau, lse_pert=lp2) if with_noise else dict(lse=lp2)
+    ops.attention_with_stats(qd, kd, vd, o1, scale, causal, a1, a2, **kw32)
+    ops.attention_with_stats_half(qd, kd, vd, o2, scale, causal, h1, h2, **kw16)
+    torch.cuda.synchronize()
+    assert torch.equal(o1, o2) and torch.equal(lp1, lp2)
+    assert torch.equal(h1, a1.half()) and torch.equal(h2, a2.half())
+
+
+@pytest.mark.gpu
+def test_fp16_statistics_form_refuses_prefill_shapes():
+    from triton_amd import ops
+    q, k, v = make(1, 2, 2, 33, 64, 64)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    h1 = torch.zeros(1, 2, 64, device="cuda", dtype=torch.float16)
+    with pytest.raises(ValueError):
+        ops.attention_with_stats_half(qd, kd, vd, torch.zeros_like(qd), 0.125, True, h1)

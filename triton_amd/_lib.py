@@ -18,6 +18,7 @@ EXPORTS = (
     "trn_attn_fwd_f16", "trn_attn_colstats_f16", "trn_prenorm_qkv_f16", "trn_calibration_copy",
     "trn_calibration_mfma", "trn_attn_workspace_bytes", "trn_attn_fwd_ws_f16", "trn_linear_f16", "trn_gate_f16", "trn_attn_fwd_stats_f16",
     "trn_attn_fwd_noalloc_f16", "trn_attn_fwd_kernel_name", "trn_attn_colmeanstd_f16", "trn_attn_fwd_probs_f16",
+    "trn_attn_fwd_stats_half_f16",
 )
 
 
@@ -72,6 +73,8 @@ def load() -> C.CDLL:
     lib.trn_attn_fwd_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.trn_attn_fwd_stats_f16.restype = C.c_int
     lib.trn_attn_fwd_stats_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.trn_attn_fwd_stats_half_f16.restype = C.c_int
+    lib.trn_attn_fwd_stats_half_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.trn_linear_f16.restype = C.c_int
     lib.trn_linear_f16.argtypes = [vp, C.c_int64, C.c_int64, C.c_int64, C.c_int32, C.POINTER(vp), C.POINTER(C.c_int64),
                                    C.POINTER(C.c_int64), C.POINTER(vp), C.POINTER(C.c_int64), C.POINTER(vp), vp]

@@ -21,12 +21,15 @@ struct AttnArgs {
     float* col_sum; float* col_sumsq;
     // ... and the probabilities themselves, un-reduced: float [B, Hq, Sq, Skv] contiguous
     float* probs;
+    // decode kernel only: noise, col_sum and col_sumsq point at fp16 data (noise pitches in halfs)
+    int io16;
 };
 
 // Checks, argument block and kernel choice behind every attention entry point of the C ABI.
 int attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
                  const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
-                 int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs = nullptr);
+                 int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs = nullptr,
+                 bool io16 = false);
 
 // At most 32 queries per head (decode): one workgroup per head whose eight waves split the keys (attn_decode.hip).
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream);

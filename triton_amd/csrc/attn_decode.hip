@@ -28,9 +28,11 @@ template <int DV> __device__ __forceinline__ int swzv(int r) {
 // all of K, but streams only its DV = D / DS columns of V and writes those columns of O).  One CU pulls 40 - 55 GB/s
 // whatever its waves ask for, and with one workgroup per head that rate is what the kernel's time is made of; more
 // workgroups per head without anything to hand over between them means fewer bytes through each CU.
-template <int D, int DS, bool NOISE>
+// NZ: 0 no score perturbation, 1 fp32 noise, 2 fp16 noise
+template <int D, int DS, int NZ>
 __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs a) {
 #if defined(__HIP_DEVICE_COMPILE__)   // buffer descriptors and LDS-load builtins exist in the device pass only
+    constexpr bool NOISE = NZ != 0, N16 = NZ == 2;
     constexpr int DV = D / DS;    // columns of V / O this workgroup owns
     constexpr int NS = D / 16;    // k-steps of S^T = K Q^T
     constexpr int NSV = DV / 16;  // (2 key halves) x (DV/32) MFMAs of P V
@@ -114,15 +116,25 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     float m = -INFINITY, l = 0.f;       // running max (log2 domain, shared by the lane pair) and this lane's partial sum
     float m2 = -INFINITY, l2 = 0.f;     // the same for the perturbed scores (KeyFormer)
     // KeyFormer noise: this lane's query row, the 4 x 4 keys of its accumulator layout per block, one block ahead
+    // (fp16 noise: 8-byte pieces of 4 keys, widened as they arrive)
+    constexpr int nsz = N16 ? 2 : 4;     // bytes per noise element
     const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(NOISE ? a.noise + b * a.nb + head * a.nh : nullptr), 0,
-        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * 4) : 0, 0x00020000);
-    const int nvo = NOISE ? (int)(((int64_t)qrow_ld * a.ns + 4 * h) * 4) : 0;
+        (void*)(NOISE ? reinterpret_cast<const char*>(a.noise) + (b * a.nb + head * a.nh) * nsz : nullptr), 0,
+        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * nsz) : 0, 0x00020000);
+    const int nvo = NOISE ? (int)(((int64_t)qrow_ld * a.ns + 4 * h) * nsz) : 0;
     float4_t g0[4], g1[4];
     auto fetch_noise = [&](int blk, float4_t (&g)[4]) __attribute__((always_inline)) {
+        if constexpr (N16) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4)
-            g[r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(nrs, nvo + r4 * 32, blk * 128, 0));
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const half4_t hv = __builtin_bit_cast(half4_t, __builtin_amdgcn_raw_buffer_load_b64(nrs, nvo + r4 * 16, blk * 64, 0));
+                g[r4] = float4_t{(float)hv[0], (float)hv[1], (float)hv[2], (float)hv[3]};
+            }
+        } else {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4)
+                g[r4] = __builtin_bit_cast(float4_t, __builtin_amdgcn_raw_buffer_load_b128(nrs, nvo + r4 * 32, blk * 128, 0));
+        }
     };
 
     // this workgroup's blocks: a contiguous share of the keys when they are split over several workgroups
@@ -402,8 +414,12 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int qr = 8 * (r / 4) + 4 * h + (r % 4);
-                    g[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
-                        nrs, (int)((qr * a.ns + c) * 4), blk * 128, 0));
+                    if constexpr (N16)
+                        g[r] = (float)__builtin_bit_cast(half_t, __builtin_amdgcn_raw_buffer_load_b16(
+                            nrs, (int)((qr * a.ns + c) * 2), blk * 64, 0));
+                    else
+                        g[r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                            nrs, (int)((qr * a.ns + c) * 4), blk * 128, 0));
                 }
             }
         };
@@ -434,8 +450,14 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             }
             x = half_sum(x); y = half_sum(y);
             if (h == 0 && key < a.Skv) {
-                if (a.col_sum) a.col_sum[(int64_t)bh * a.Skv + key] = x;
-                if (a.col_sumsq) a.col_sumsq[(int64_t)bh * a.Skv + key] = y;
+                const int64_t at = (int64_t)bh * a.Skv + key;
+                if (a.io16) {       // (the fp32 value rounded once, as a copy into the caller's fp16 tensor would)
+                    if (a.col_sum) reinterpret_cast<half_t*>(a.col_sum)[at] = (half_t)x;
+                    if (a.col_sumsq) reinterpret_cast<half_t*>(a.col_sumsq)[at] = (half_t)y;
+                } else {
+                    if (a.col_sum) a.col_sum[at] = x;
+                    if (a.col_sumsq) a.col_sumsq[at] = y;
+                }
             }
         };
         const int first = dsl * DNW + wave;
@@ -483,12 +505,12 @@ static int decode_col_shares(int64_t n_bh, int seq_kv, int head_dim) {
 const char* attn_decode_kernel_name(int batch, int n_q_heads, int seq_kv, int head_dim, bool noise) {
     const int ds = decode_col_shares((int64_t)batch * n_q_heads, seq_kv, head_dim);
     if (head_dim == 128) {
-        if (ds == 4) return noise ? "trn::attn_decode_kernel<128, 4, true>" : "trn::attn_decode_kernel<128, 4, false>";
-        if (ds == 2) return noise ? "trn::attn_decode_kernel<128, 2, true>" : "trn::attn_decode_kernel<128, 2, false>";
-        return noise ? "trn::attn_decode_kernel<128, 1, true>" : "trn::attn_decode_kernel<128, 1, false>";
+        if (ds == 4) return noise ? "trn::attn_decode_kernel<128, 4, 1>" : "trn::attn_decode_kernel<128, 4, 0>";
+        if (ds == 2) return noise ? "trn::attn_decode_kernel<128, 2, 1>" : "trn::attn_decode_kernel<128, 2, 0>";
+        return noise ? "trn::attn_decode_kernel<128, 1, 1>" : "trn::attn_decode_kernel<128, 1, 0>";
     }
-    if (ds == 2) return noise ? "trn::attn_decode_kernel<64, 2, true>" : "trn::attn_decode_kernel<64, 2, false>";
-    return noise ? "trn::attn_decode_kernel<64, 1, true>" : "trn::attn_decode_kernel<64, 1, false>";
+    if (ds == 2) return noise ? "trn::attn_decode_kernel<64, 2, 1>" : "trn::attn_decode_kernel<64, 2, 0>";
+    return noise ? "trn::attn_decode_kernel<64, 1, 1>" : "trn::attn_decode_kernel<64, 1, 0>";
 }
 
 hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t workspace_bytes, hipStream_t stream) {
@@ -507,13 +529,10 @@ hipError_t launch_attn_decode(AttnArgs a, int head_dim, void* workspace, int64_t
     if (grid > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 g((unsigned)grid), t(DNW * 64);
 #define TRN_DEC(D_, DS_, N_) hipLaunchKernelGGL((attn_decode_kernel<D_, DS_, N_>), g, t, 0, stream, a)
-    if (a.noise) {
-        if (head_dim == 128) { if (ds == 4) TRN_DEC(128, 4, true); else if (ds == 2) TRN_DEC(128, 2, true); else TRN_DEC(128, 1, true); }
-        else { if (ds == 2) TRN_DEC(64, 2, true); else TRN_DEC(64, 1, true); }
-    } else {
-        if (head_dim == 128) { if (ds == 4) TRN_DEC(128, 4, false); else if (ds == 2) TRN_DEC(128, 2, false); else TRN_DEC(128, 1, false); }
-        else { if (ds == 2) TRN_DEC(64, 2, false); else TRN_DEC(64, 1, false); }
-    }
+#define TRN_DEC_NZ(D_, DS_) do { if (!a.noise) TRN_DEC(D_, DS_, 0); else if (a.io16) TRN_DEC(D_, DS_, 2); else TRN_DEC(D_, DS_, 1); } while (0)
+    if (head_dim == 128) { if (ds == 4) TRN_DEC_NZ(128, 4); else if (ds == 2) TRN_DEC_NZ(128, 2); else TRN_DEC_NZ(128, 1); }
+    else { if (ds == 2) TRN_DEC_NZ(64, 2); else TRN_DEC_NZ(64, 1); }
+#undef TRN_DEC_NZ
 #undef TRN_DEC
     return hipGetLastError();
 }

@@ -476,9 +476,21 @@ extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, con
     return trn_attn_colstats_f16(d, q, k, rows, noise, out_sum, out_sumsq, stream);
 }
 
+extern "C" int trn_attn_fwd_stats_half_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                           float* lse, const void* gamma_q, const void* noise, float* lse_pert,
+                                           void* out_sum, void* out_sumsq, void* stream) {
+    using namespace trn;
+    if (!d) return TRN_E_NULL;
+    if (!out_sum && !out_sumsq) return TRN_E_NULL;
+    if (d->q_norm || d->seq_q > 32) return TRN_E_UNSUPPORTED;
+    return attn_forward(d, q, k, v, o, lse, gamma_q, static_cast<const float*>(noise), lse_pert, nullptr, 0,
+                        static_cast<float*>(out_sum), static_cast<float*>(out_sumsq), stream, nullptr, true);
+}
+
 int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o, float* lse,
                              const void* gamma_q, const float* noise, float* lse_pert, void* workspace,
-                             int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs) {
+                             int64_t workspace_bytes, float* col_sum, float* col_sumsq, void* stream, float* probs,
+                             bool io16) {
     if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;
     if (!d || !q || !k || !v || !o) return TRN_E_NULL;
     if (noise && !lse_pert) return TRN_E_NULL;
@@ -491,10 +503,14 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
         if (d->noise_stride_s < d->seq_kv) return TRN_E_STRIDE;
         // one head's noise is addressed with 32-bit byte offsets
         if ((int64_t)d->seq_q * d->noise_stride_s * 4 + 1024 > 0x7fffffffLL) return TRN_E_UNSUPPORTED;
-        if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
-            !pitch16(d->noise_stride_b, 4))
+        if (io16) {     // fp16 noise is fetched 8 bytes at a time
+            if ((reinterpret_cast<uintptr_t>(noise) & 7u) || (d->noise_stride_s & 3) || (d->noise_stride_h & 3) || (d->noise_stride_b & 3))
+                return TRN_E_ALIGN;
+        } else if (!aligned16(noise) || !pitch16(d->noise_stride_s, 4) || !pitch16(d->noise_stride_h, 4) ||
+                   !pitch16(d->noise_stride_b, 4))
             return TRN_E_ALIGN;
     }
+    if (io16 && d->seq_q > 32) return TRN_E_UNSUPPORTED;     // fp16 noise and statistics: the decode kernel only
     AttnArgs a;
     a.q = (const half_t*)q; a.k = (const half_t*)k; a.v = (const half_t*)v; a.o = (half_t*)o;
     a.lse = lse; a.gamma_q = (const half_t*)gamma_q; a.noise = noise; a.lse_pert = lse_pert;
@@ -509,7 +525,7 @@ int trn::attn_forward(const trn_attn_desc* d, const void* q, const void* k, cons
     const float tau = noise ? d->tau : 1.f;
     a.c2 = d->scale * kLog2e / tau; a.c3 = kLog2e / tau;
     a.q_eps = d->q_norm_eps; a.causal = d->causal ? 1 : 0; a.q_norm = d->q_norm ? 1 : 0;
-    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs;
+    a.n_split = 1; a.ws = nullptr; a.col_sum = col_sum; a.col_sumsq = col_sumsq; a.probs = probs; a.io16 = io16 ? 1 : 0;
     // K/V tiles are fetched with 32-bit buffer offsets relative to the (batch, head) base
     // (with room for the blocks the pipelines request past the end, which must stay representable to read as zeros)
     if (((int64_t)d->seq_kv + 2048) * d->k_stride_s * 2 > 0x7fffffffLL || ((int64_t)d->seq_kv + 2048) * d->v_stride_s * 2 > 0x7fffffffLL)

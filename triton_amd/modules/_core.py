@@ -113,6 +113,17 @@ def _noise_fp32(mod: "FusedModule", n4: torch.Tensor) -> torch.Tensor:
     return view
 
 
+def _half_io_ok(t: torch.Tensor, shape) -> bool:
+    """A caller-owned fp16 statistics tensor that the kernel can write directly."""
+    return t.dtype == torch.float16 and t.is_contiguous() and tuple(t.shape) == tuple(shape)
+
+
+def _half_noise_ok(n3: torch.Tensor) -> bool:
+    """fp16 noise [H, M, P+M] that the decode kernel can read as it is (8-byte pieces)."""
+    return (n3.dtype == torch.float16 and n3.dim() == 3 and n3.stride(2) == 1 and n3.data_ptr() % 8 == 0
+            and n3.stride(0) % 4 == 0 and n3.stride(1) % 4 == 0)
+
+
 def _store_scores(dst: torch.Tensor, src32: torch.Tensor) -> None:
     """Key scores are produced in fp32; a caller-owned fp16 tensor (the reference allocates every
     tensor as fp16, vanilla_llama_benchmark.py:131-139) receives them rounded."""
@@ -334,8 +345,14 @@ class DecodeKeyFormer(_DecodeAppend):
         q, _ = self._project(X, WQ, WK, WV, K_cache, V_cache)
         H, M, D = q.shape
         PM = K_cache.shape[1]
-        n4 = _noise_fp32(self, noise[None])
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
+        if self.reduce and M <= 32 and _half_io_ok(C_out, (H, PM)) and _half_noise_ok(noise):
+            # everything fp16 as the reference's drivers allocate it: one launch, no copies on the side
+            ops.attention_with_stats_half(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale,
+                                          self.causal, C_out.view(1, H, PM), None, noise=noise[None], tau=self.tau,
+                                          lse_pert=lsep)
+            return
+        n4 = _noise_fp32(self, noise[None])
         shape = (1, H, PM) if self.reduce else (1, H, M, PM)
         if C_out.numel() != H * PM * (1 if self.reduce else M):
             raise ValueError(f"C_out {tuple(C_out.shape)}: expected {shape[1:]}")
@@ -361,6 +378,10 @@ class DecodeRoCo(_DecodeAppend):
         H, M, D = q.shape
         PM = K_cache.shape[1]
         lse = self._workspace("lse", (1, H, M), torch.float32, X.device)
+        if M <= 32 and _half_io_ok(C_out1, (H, PM)) and _half_io_ok(C_out2, (H, PM)):
+            ops.attention_with_stats_half(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale,
+                                          self.causal, C_out1.view(1, H, PM), C_out2.view(1, H, PM), lse=lse)
+            return
         outs = []
         for i, c in enumerate((C_out1, C_out2)):
             outs.append(c.view(1, H, PM) if c.dtype == torch.float32 and c.is_contiguous() else

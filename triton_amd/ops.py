@@ -91,7 +91,10 @@ def _attn_desc(q, k, v, o, scale, causal, q_norm, q_eps, noise, tau) -> _lib.Att
     d.scale, d.causal = float(scale), int(bool(causal))
     d.q_norm, d.q_norm_eps = int(bool(q_norm)), float(q_eps)
     if noise is not None:
-        _dev_float(noise, "noise")
+        if noise.dtype == torch.float16:        # (only trn_attn_fwd_stats_half_f16 takes it; the strides count halfs)
+            _dev_half(noise, "noise")
+        else:
+            _dev_float(noise, "noise")
         _need(tuple(noise.shape) == (B, Hq, Sq, Skv), f"noise {tuple(noise.shape)}: expected {(B, Hq, Sq, Skv)}")
         d.noise_stride_b, d.noise_stride_h, d.noise_stride_s = noise.stride(0), noise.stride(1), noise.stride(2)
     d.tau = float(tau)
@@ -220,6 +223,31 @@ def attention_with_stats(q, k, v, o, scale: float, causal: bool, out_sum: Option
     st = lib.trn_attn_fwd_stats_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), None, _ptr(noise),
                                     _ptr(lse_pert), _ptr(out_sum), _ptr(out_sumsq), _stream(q))
     _lib.check("trn_attn_fwd_stats_f16", st)
+
+
+def attention_with_stats_half(q, k, v, o, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
+                              out_sumsq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
+                              noise: Optional[torch.Tensor] = None, tau: float = 1.0,
+                              lse_pert: Optional[torch.Tensor] = None) -> None:
+    """`attention_with_stats` for at most 32 queries per head with fp16 noise and fp16 statistics, as the reference's
+    drivers allocate them: one launch, nothing widened or narrowed on the side."""
+    _need(noise is None or noise.dtype == torch.float16, "noise: expected float16")
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, noise, tau)
+    B, Hq, Sq, _ = q.shape
+    Skv = k.shape[2]
+    _need(Sq <= 32, f"{Sq} queries per head: the fp16 form is for at most 32")
+    _row_stat(lse, "lse", (B, Hq, Sq)); _row_stat(lse_pert, "lse_pert", (B, Hq, Sq))
+    for t, n in ((out_sum, "out_sum"), (out_sumsq, "out_sumsq")):
+        if t is not None:
+            _dev_half(t, n)
+            _need(tuple(t.shape) == (B, Hq, Skv) and t.is_contiguous(), f"{n}: expected contiguous float16 {(B, Hq, Skv)}")
+    _need(out_sum is not None or out_sumsq is not None, "no statistics output given")
+    if noise is not None:
+        _need(lse_pert is not None, "noise requires lse_pert")
+    lib = _lib.load()
+    st = lib.trn_attn_fwd_stats_half_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), None, _ptr(noise),
+                                         _ptr(lse_pert), _ptr(out_sum), _ptr(out_sumsq), _stream(q))
+    _lib.check("trn_attn_fwd_stats_half_f16", st)
 
 
 def prenorm_qkv(x: torch.Tensor, gamma: Optional[torch.Tensor], wq, wk, wv, q_out, k_out, v_out,
