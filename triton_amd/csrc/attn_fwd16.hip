@@ -38,6 +38,7 @@ __device__ __forceinline__ float4_t mfma16(half8_t a, half8_t b, float4_t c) {
 __device__ __forceinline__ void swap_rows16(float& a, float& b) {
     asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
 }
+__device__ __forceinline__ int imax3(int a, int b, int c) { return max(max(a, b), c); }
 __device__ __forceinline__ float quad_max(float x) { float a = x, b = x; swap_rows16(a, b); return half_max(fmaxf(a, b)); }
 __device__ __forceinline__ float quad_sum(float x) { float a = x, b = x; swap_rows16(a, b); return half_sum(a + b); }
 
@@ -104,42 +105,7 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     int qrow[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) qrow[qb] = wq0 + 16 * qb + n;
-
-    // ---- Q^T B-operands: lane holds Q[qrow[qb]][32 ks + 8 g4 .. +7]
     half8_t qB[2][NKS];
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-        const int qrow_ld = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;       // clamp loads; stores are predicated
-        const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * g4;
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) qB[qb][ks] = *reinterpret_cast<const half8_t*>(qp + ks * 32);
-        const bool q_norm = a.q_norm != 0;
-        if (q_norm) {   // fused per-head RMSNorm of the query row (the rest of the row is in the lanes n + 16, + 32, + 48)
-            float ss = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks)
-#pragma unroll
-                for (int e = 0; e < 8; ++e) { float f = (float)qB[qb][ks][e]; ss += f * f; }
-            ss = quad_sum(ss);
-            const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
-#pragma unroll
-            for (int ks = 0; ks < NKS; ++ks) {
-                half8_t gq;
-                if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 32 + 8 * g4);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) {
-                    float y = (float)qB[qb][ks][e] * rstd;
-                    if (a.gamma_q) y = (float)gq[e] * y;
-                    qB[qb][ks][e] = (half_t)y;
-                }
-            }
-        }
-        // the softmax scale and log2(e) go into Q once, so that the scores leave the matrix pipe ready for exp2
-#pragma unroll
-        for (int ks = 0; ks < NKS; ++ks)
-#pragma unroll
-            for (int e = 0; e < 8; ++e) qB[qb][ks][e] = (half_t)((float)qB[qb][ks][e] * a.c1);
-    }
 
     // ---- LDS read offsets (halfs).  K operand (ks, kb): row 16 kb + n of a 32-key block, logical chunk 4 ks + g4
     // (the swizzle depends on the row's low four bits only, so the second key half is a constant 16 rows further).
@@ -187,55 +153,67 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
     const int wb = wq0 + off;          // key index bound of this wave's first query
     auto needs_mask = [&](int key0) { return (key0 + 32 > a.Skv) || (a.causal && key0 + 31 > wb); };
 
-    // Scores of a 32-key block starting at key0, just produced: mask; the lane's own maximum per query against the
-    // lazy reference m (raised only when some score exceeds it by more than 2^8: see attn_fwd.hip).  Returns
-    // whether a rescale is due (wave-uniform) and the lane's candidate maxima.
-    auto reduce_block = [&](bool masked, Scores16& sx, int key0, float (&smax)[2]) __attribute__((always_inline)) {
-        if (masked) {
+    // Scores of a 32-key block starting at key0, just produced: keys past the end and, under a causal mask, keys
+    // after the query become -inf.
+    auto mask_block = [&](Scores16& sx, int key0) __attribute__((always_inline)) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+        for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int qb = 0; qb < 2; ++qb)
+            for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const int key = key0 + 16 * kb + 4 * g4 + i;
-                        const bool ok = key < a.Skv && (!a.causal || key <= qrow[qb] + off);
-                        sx.s[kb][qb][i] = ok ? sx.s[kb][qb][i] : -INFINITY;
-                    }
-        }
-        bool over = false;
+                for (int i = 0; i < 4; ++i) {
+                    const int key = key0 + 16 * kb + 4 * g4 + i;
+                    const bool ok = key < a.Skv && (!a.causal || key <= qrow[qb] + off);
+                    sx.s[kb][qb][i] = ok ? sx.s[kb][qb][i] : -INFINITY;
+                }
+    };
+    // The lane's maximum per query over its 8 keys of the block.
+    auto block_max = [&](const Scores16& sx, float (&smax)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const float4_t& u = sx.s[0][qb];
             const float4_t& w = sx.s[1][qb];
             smax[qb] = fmaxf(max3(u[0], u[1], u[2]), max3(u[3], w[0], w[1]));
             smax[qb] = max3(smax[qb], w[2], w[3]);
-            over = over || smax[qb] > 8.0f;
         }
-        return __builtin_amdgcn_ballot_w64(over) != 0;
     };
-    // smax is relative to m, and so are the scores sx already in flight: they move with it
-    auto rescale = [&](const float (&smax)[2], Scores16& sx) __attribute__((always_inline)) {
+    // Is a rescale due?  The reference m is lazy (raised only when some score exceeds it by more than 2^8: see
+    // attn_fwd.hip), the scores arrive relative to it, and the decision is wave-uniform, so only whether any of the
+    // lane's 16 scores exceeds 8 matters.  For that the bit patterns will do: non-negative floats order as signed
+    // integers and every negative float (masked scores included) lies below them.  One three-way integer maximum per
+    // two scores, both queries of the lane together, no canonicalising of the operands (9 vector instructions per block
+    // against 15 for two float maxima); the per-query maxima are formed on the rare path only.  In four pieces, one per
+    // accumulator quad, so that they sit behind four different MFMAs.
+    auto max_piece = [&](const Scores16& sx, int piece, int mx) __attribute__((always_inline)) {
+        const float4_t& u = sx.s[piece >> 1][piece & 1];
+        if (piece == 0) return max(imax3(__float_as_int(u[0]), __float_as_int(u[1]), __float_as_int(u[2])), __float_as_int(u[3]));
+        mx = imax3(mx, __float_as_int(u[0]), __float_as_int(u[1]));
+        return imax3(mx, __float_as_int(u[2]), __float_as_int(u[3]));
+    };
+    // the scores sx already in flight are relative to m: they move with it
+    auto rescale = [&](Scores16& sx) __attribute__((always_inline)) {
+        float smax[2];
+        block_max(sx, smax);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             const float up = fmaxf(0.f, quad_max(smax[qb]));
-            const float mnew = m[qb] + up;
             const float alpha = fast_exp2(-up);
             sx.s[0][qb] = sx.s[0][qb] - up;
             sx.s[1][qb] = sx.s[1][qb] - up;
-            negm[qb] = float4_t{-mnew, -mnew, -mnew, -mnew};
+            negm[qb] = negm[qb] - up;                   // (in place, like the accumulators: a fresh vector here makes
+                                                        // the path that skips the rescale copy it every block)
             lacc[qb] = lacc[qb] * alpha;
 #pragma unroll
             for (int i = 0; i < NOP; ++i)
                 oacc[i][qb] = oacc[i][qb] * alpha;      // (as one vector operation: written per element, the path that
                                                         // skips the rescale ends up copying every accumulator)
-            m[qb] = mnew;
+            m[qb] = m[qb] + up;
         }
     };
 
     const half_t one = (half_t)1.f;
     const half8_t ones8 = {one, one, one, one, one, one, one, one};
-    constexpr int NQ = 2;   // operand look-ahead, in operands (= 2 NQ MFMA slots; 4 measured no better)
+    constexpr int NQ = 2;   // operand look-ahead, in operands (= 2 NQ MFMA slots; 4 measured no better, twice)
     static_assert(NOP % NQ == 0, "the operand window must divide the operands of a phase");
     half8_t ka[NQ];    // K operands of the next block's S^T, a rolling window ahead of use
     half8_t va[NQ];    // V^T operands of this block's P V, likewise
@@ -287,8 +265,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
             __builtin_amdgcn_sched_barrier(0);
         }
         // ---- phase B ----
-        float smax[2] = {0.f, 0.f};
         bool due = false;
+        int mx = 0;
 #pragma unroll
         for (int i = 0; i < NS; ++i) {
             const int db = i >> 1, qb = i & 1;
@@ -297,18 +275,61 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
                 if (db + NQ < NOP) load_v(db + NQ, db % NQ);
                 else load_k(K2, db + NQ - NOP, db % NQ);
             }
-            if (i == NS / 2) due = reduce_block(MAYMASK && masked_next, sn, key0_next, smax);
+            constexpr int R0 = NS / 2 - (NS >= 16 ? 3 : 2);
+            if (i == R0) { if (MAYMASK && masked_next) mask_block(sn, key0_next); }
+            if (i >= R0 && i < R0 + 4) mx = max_piece(sn, i - R0, mx);
+            if (i == R0 + 3) due = __builtin_amdgcn_ballot_w64(mx > 0x41000000) != 0;       // 8.0f
             __builtin_amdgcn_sched_barrier(0);
         }
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) lacc[qb] = mfma16(ones8, pB[qb], lacc[qb]);
-        if (due) rescale(smax, sn);
+        if (due) rescale(sn);
     };
 
     // ---- prologue: K stages 0 and 1 and V stage 0; scores of block 0; first K operands of block 1 ----
     TRN_FETCH_K(0, Ks0);
     TRN_FETCH_V(0, Vs0);
     if (ntiles > 1) TRN_FETCH_K(1, Ks1);
+
+    // ---- Q^T B-operands: lane holds Q[qrow[qb]][32 ks + 8 g4 .. +7].  The loads go out behind the first K/V stage
+    // fetches and all together, so that the workgroup's start-up pays one memory latency, not three in a row.
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        const int qrow_ld = qrow[qb] < a.Sq ? qrow[qb] : a.Sq - 1;       // clamp loads; stores are predicated
+        const half_t* qp = a.q + b * a.qb + head * a.qh + (int64_t)qrow_ld * a.qs + 8 * g4;
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks) qB[qb][ks] = *reinterpret_cast<const half8_t*>(qp + ks * 32);
+    }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        const bool q_norm = a.q_norm != 0;
+        if (q_norm) {   // fused per-head RMSNorm of the query row (the rest of the row is in the lanes n + 16, + 32, + 48)
+            float ss = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) { float f = (float)qB[qb][ks][e]; ss += f * f; }
+            ss = quad_sum(ss);
+            const float rstd = 1.0f / __builtin_sqrtf(ss / (float)D + a.q_eps);
+#pragma unroll
+            for (int ks = 0; ks < NKS; ++ks) {
+                half8_t gq;
+                if (a.gamma_q) gq = *reinterpret_cast<const half8_t*>(a.gamma_q + ks * 32 + 8 * g4);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    float y = (float)qB[qb][ks][e] * rstd;
+                    if (a.gamma_q) y = (float)gq[e] * y;
+                    qB[qb][ks][e] = (half_t)y;
+                }
+            }
+        }
+        // the softmax scale and log2(e) go into Q once, so that the scores leave the matrix pipe ready for exp2
+#pragma unroll
+        for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) qB[qb][ks][e] = (half_t)((float)qB[qb][ks][e] * a.c1);
+    }
+
     __builtin_amdgcn_s_waitcnt(0x0f70);     // vmcnt(0): this wave's loads have landed in LDS
     __syncthreads();
 
@@ -326,7 +347,8 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd16_kernel(co
         for (int i = 0; i < NQ; ++i) load_k(Ks0 + 32 * D, i, i);
         // block 0 sets the reference outright (every query sees key 0, so it is finite from here on)
         float smax[2];
-        reduce_block(true, sA, 0, smax);
+        mask_block(sA, 0);
+        block_max(sA, smax);
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) {
             m[qb] = quad_max(smax[qb]);

@@ -2,7 +2,14 @@
 summary: per-kernel call counts and average durations (`--kernel-trace --stats` runs) and per-kernel
 counter values averaged per dispatch (`--pmc` runs).
 
-    python -m triton_amd.profiling /tmp/prof/attn_results.db [--filter trn::] [--calib-bytes N]
+    python -m triton_amd.profiling /tmp/prof/attn_results.db [--filter trn::] [--calib-bytes N] [--bench-json FILE]
+
+Durations are given three ways: the plain average over every dispatch, the median, and the mean over the
+dispatches that start later than --settle seconds (default 0.25) after the first dispatch of the trace.  The
+plain average includes the cold call, the warm-ups and the first tens of milliseconds of a burst, during
+which the board's clocks are still rising; the other two are the steady state that `bench.py` times.  With
+--bench-json FILE (the JSON line `bench.py` printed in the profiled run) the header repeats that line's
+ms_per_step and kernel_ms, so that the trace and the bench of one run on one board can be read side by side.
 
 With --calib-bytes N the FETCH_SIZE / WRITE_SIZE readings (KiB per dispatch) of every kernel are also
 shown scaled by what the library's calibration copy kernel read for its known N bytes.
@@ -19,14 +26,28 @@ def short(name: str) -> str:
     return name[-72:]
 
 
-def kernel_stats(con):
-    """(name, calls, total ns, average ns) per kernel from the dispatch trace."""
+def kernel_stats(con, settle_s: float = 0.25):
+    """(name, calls, total ns, average ns, median ns, steady-state mean ns, steady-state calls) per kernel from the
+    dispatch trace; steady state = dispatches starting more than settle_s after the trace's first dispatch."""
     try:
-        rows = list(con.execute("select name, count(*), sum(end - start), avg(end - start) from kernels "
-                                "group by name order by sum(end - start) desc"))
+        rows = list(con.execute("select name, start, end from kernels order by start"))
     except sqlite3.Error:
         return []
-    return rows
+    if not rows:
+        return []
+    t0 = rows[0][1]
+    per = collections.defaultdict(list)
+    for name, start, end in rows:
+        per[name].append((start, end - start))
+    out = []
+    for name, ds in per.items():
+        durs = sorted(d for _, d in ds)
+        steady = [d for st, d in ds if st - t0 > settle_s * 1e9]
+        total = sum(durs)
+        out.append((name, len(durs), total, total / len(durs), durs[len(durs) // 2],
+                    sum(steady) / len(steady) if steady else float("nan"), len(steady)))
+    out.sort(key=lambda r: -r[2])
+    return out
 
 
 def counters(con):
@@ -57,13 +78,24 @@ def main():
     ap.add_argument("db")
     ap.add_argument("--filter", default="trn", help="only kernels whose name contains this (default: this library's)")
     ap.add_argument("--calib-bytes", type=int, default=0)
+    ap.add_argument("--settle", type=float, default=0.25, help="seconds after the first dispatch that count as warm-up")
+    ap.add_argument("--bench-json", default="", help="file holding the JSON line bench.py printed in the profiled run")
     a = ap.parse_args()
+    if a.bench_json:
+        import json
+        with open(a.bench_json) as f:
+            lines = [ln for ln in f.read().splitlines() if ln.startswith("{")]
+        if lines:
+            b = json.loads(lines[-1])
+            r = b.get("roofline", {})
+            print(f"bench.py line of this run: ms_per_step {b.get('ms_per_step')}  roofline.kernel_ms {r.get('kernel_ms')}  "
+                  f"roofline.achieved {r.get('achieved')} {r.get('unit')}  frac {r.get('frac')}  kernel {r.get('kernel')}")
     con = sqlite3.connect(a.db)
-    stats = [r for r in kernel_stats(con) if a.filter in r[0]]
+    stats = [r for r in kernel_stats(con, a.settle) if a.filter in r[0]]
     if stats:
-        print(f"{'kernel':72s} {'calls':>6s} {'avg_us':>10s} {'total_us':>11s}")
-        for name, calls, total, avg in stats:
-            print(f"{short(name):72s} {calls:6d} {avg / 1e3:10.2f} {total / 1e3:11.1f}")
+        print(f"{'kernel':72s} {'calls':>6s} {'avg_us':>10s} {'median_us':>10s} {'steady_us':>10s} {'(calls)':>8s} {'total_us':>11s}")
+        for name, calls, total, avg, med, steady, nst in stats:
+            print(f"{short(name):72s} {calls:6d} {avg / 1e3:10.2f} {med / 1e3:10.2f} {steady / 1e3:10.2f} {nst:8d} {total / 1e3:11.1f}")
     agg, disp, dur, bygrid, gdisp = counters(con)
     calib = {}
     for (name, grid), vals in bygrid.items():       # the copy launched on exactly --calib-bytes (16 bytes per work-item)
