@@ -1,5 +1,6 @@
 """GPU parity for the key-score paths: forward (row LSE) + trn_attn_colstats_f16, against the CPU oracle.
-fp32 key scores: 1e-3 relative (plus 1e-5 absolute for near-zero columns)."""
+fp32 key scores: 1e-3 relative.  The absolute allowance is 1e-9: sums of squares of late keys are of order 1e-6 and
+below, and a larger allowance would leave exactly those columns unchecked."""
 import pytest
 import torch
 
@@ -8,7 +9,7 @@ from oracle import ref
 pytestmark = pytest.mark.gpu
 
 
-def close_scores(got, want, rtol=1e-3, atol=1e-5):
+def close_scores(got, want, rtol=1e-3, atol=1e-9):
     got = got.float().cpu(); want = want.float()
     err = (got - want).abs()
     bad = err > atol + rtol * want.abs()

@@ -246,7 +246,10 @@ __global__ __launch_bounds__(256, NOISE ? 2 : 3) void attn_colstats_kernel(const
             // n = queries that see this key: all of them, or under a causal mask those from key - (Skv - Sq) on
             const float n = (float)(a.causal ? a.Sq - max(0, key - (a.Skv - a.Sq)) : a.Sq);
             const float mean = x / n;
-            y = __builtin_sqrtf(fmaxf(0.f, y / n - mean * mean));
+            // E p^2 - mean^2 as (y - x mean) / n, the product fused.  The difference is known to about 1e-7 of E p^2, its
+            // root to 3e-4 of the column's root mean square: a key seen by a single query, whose spread is zero by
+            // definition, would come back as that rounding residue, so it is set.
+            y = n > 1.5f ? __builtin_sqrtf(fmaxf(0.f, __builtin_fmaf(-x, mean, y) / n)) : 0.f;
             x = mean;
         }
         if (c == 0 && key < a.Skv) {
@@ -467,7 +470,10 @@ __global__ __launch_bounds__(256, 2) void attn_colstats_plain_kernel(const ColAr
             // n = queries that see this key: all of them, or under a causal mask those from key - (Skv - Sq) on
             const float n = (float)(a.causal ? a.Sq - max(0, key - (a.Skv - a.Sq)) : a.Sq);
             const float mean = x / n;
-            y = __builtin_sqrtf(fmaxf(0.f, y / n - mean * mean));
+            // E p^2 - mean^2 as (y - x mean) / n, the product fused.  The difference is known to about 1e-7 of E p^2, its
+            // root to 3e-4 of the column's root mean square: a key seen by a single query, whose spread is zero by
+            // definition, would come back as that rounding residue, so it is set.
+            y = n > 1.5f ? __builtin_sqrtf(fmaxf(0.f, __builtin_fmaf(-x, mean, y) / n)) : 0.f;
             x = mean;
         }
         if (c == 0 && key < a.Skv) {
