@@ -132,7 +132,10 @@ int trn_attn_fwd_ws_f16(const trn_attn_desc* desc, const void* q, const void* k,
  * loops, harnesses that forbid hipMalloc): it has no counterpart in the reference.  The workspace is a static device
  * array inside the library, TRN_ATTN_NOALLOC_SCRATCH_BYTES per GPU, held from load until the process ends; the call
  * itself allocates and frees nothing.  A problem whose workspace (trn_attn_workspace_bytes) would be larger is
- * rejected with TRN_E_SCRATCH; one that needs none runs as trn_attn_fwd_f16.  The arrival counters are cleared by a
+ * rejected with TRN_E_SCRATCH; one that needs none runs as trn_attn_fwd_f16.  (With the present split rule -- at most
+ * 256 shares over all heads, 32 x (head_dim + 4) floats each, head_dim <= 128 -- no workspace exceeds 4.4 MB, so the
+ * rejection cannot occur today; it guards a future rule, and a host-side test sweeps trn_attn_workspace_bytes over the
+ * supported shapes against the array's size.)  The arrival counters are cleared by a
  * small kernel on `stream` before the attention kernel, so a call does not depend on what the previous one left.
  * All calls on one GPU share the one array: calls that overlap on a GPU (two streams, two threads) race; serialise
  * them, or give overlapping callers their own workspace through trn_attn_fwd_ws_f16.  Call trn_check_device once

@@ -150,6 +150,28 @@ def test_validation_of_the_workspace_statistics_and_linear_entry_points(lib):
     assert gate(c1=None) == -1 and gate(rows=0) == 0
 
 
+def test_no_workspace_exceeds_the_static_scratch_array(lib):
+    """trn_attn_fwd_noalloc_f16 rejects a problem whose workspace is larger than the library's static array.  With
+    the present split rule that cannot happen; this sweep of trn_attn_workspace_bytes over the decode shapes (host
+    arithmetic, nothing is launched) is what trips when a change to the rule makes it possible."""
+    import re
+    hdr = open(os.path.join(ROOT, "include", "trinity_hip.h")).read()
+    m = re.search(r"#define TRN_ATTN_NOALLOC_SCRATCH_BYTES \((\d+)u << (\d+)\)", hdr)
+    capacity = int(m.group(1)) << int(m.group(2))
+    largest = 0
+    for D in (64, 128):
+        for heads in (1, 2, 3, 7, 8, 16, 31, 32, 63, 64, 71, 100, 127, 128, 200):
+            for batch in (1, 2, 5):
+                for sq in (1, 16, 32):
+                    for skv in (64, 1024, 1040, 4112, 16384, 131072, 1 << 20):
+                        d = _desc(batch=batch, n_q_heads=heads, n_kv_heads=1, seq_q=sq, seq_kv=skv, head_dim=D,
+                                  q_stride_b=heads * sq * D, q_stride_h=sq * D, q_stride_s=D, k_stride_b=skv * D,
+                                  k_stride_h=skv * D, k_stride_s=D, v_stride_b=skv * D, v_stride_h=skv * D, v_stride_s=D,
+                                  o_stride_b=heads * sq * D, o_stride_h=sq * D, o_stride_s=D, causal=0)
+                        largest = max(largest, lib.trn_attn_workspace_bytes(C.byref(d)))
+    assert 0 < largest <= capacity, (largest, capacity)
+
+
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     from triton_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)

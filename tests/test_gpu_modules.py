@@ -196,6 +196,50 @@ def test_decode_append_modules_match_reference_classes(amp, M, N, D, P):
     close(t["O2"], ref.flatten_token_major(wo), atol); close(t["C_out1"], s1, 1e-6, srt); close(t["C_out2"], s2, 1e-8, srt)
 
 
+@pytest.mark.parametrize("variant", ["vanilla", "keyformer", "roco"])
+def test_decode_modules_driven_the_old_way_eagerly_with_block_keywords(variant):
+    """The older drivers' call shape (rms_benchmark.py:247-265): no graph, every call eager on the current stream,
+    block sizes passed by keyword (block_k=..., block_p=...) -- and, as convert_eval_rms.py:275-285 does it,
+    positionally after the tensors.  Both must run the same kernels as the bare call and give the oracle's result."""
+    from triton_amd import modules
+    M, N, D, P = 16, 1024, 128, 200
+    cpu, H = _decode_tensors(M, N, D, P, seed=7)
+    W = (cpu["WQ"], cpu["WK"], cpu["WV"])
+    m = modules.get(variant, "decode", head_dim=D)
+
+    def fresh():
+        t = {k: v.cuda() for k, v in cpu.items()}
+        t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+        t["C_out"] = torch.zeros(H, P + M, dtype=torch.float16, device="cuda")
+        t["C_out1"] = torch.zeros(H, P + M, device="cuda"); t["C_out2"] = torch.zeros(H, P + M, device="cuda")
+        return t
+
+    outs = {}
+    for how in ("keywords", "positional"):
+        t = fresh()
+        args = [t[p] for p in m.TENSOR_PARAMS]
+        for _ in range(3):                                  # the driver's warm-up and timed calls are all eager
+            if how == "keywords":
+                assert m.forward(*args, block_k=32, block_p=64, block_n=16) is None
+            else:
+                assert m.forward(*args, 32, 64) is None
+        torch.cuda.synchronize()
+        outs[how] = t
+    if variant == "vanilla":
+        want = ref.flatten_token_major(ref.decode_append_vanilla(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D))
+    elif variant == "keyformer":
+        wo, pw = ref.decode_append_keyformer(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], cpu["noise"], P, D, tau=1.5)
+        want = ref.flatten_token_major(wo)
+        close(outs["keywords"]["C_out"], pw.sum(dim=1), 1e-4, 2e-3)
+    else:
+        wo, s1, s2 = ref.decode_append_roco(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)
+        want = ref.flatten_token_major(wo)
+        close(outs["keywords"]["C_out1"], s1, 1e-6, 1e-3); close(outs["keywords"]["C_out2"], s2, 1e-8, 1e-3)
+    close(outs["keywords"]["O2"], want, 1e-4)
+    for name in ("O2", "C_out", "C_out1", "C_out2", "K_cache", "V_cache"):
+        assert torch.equal(outs["keywords"][name], outs["positional"][name]), name
+
+
 @pytest.mark.parametrize("variant", ["vanilla", "qknorm", "roco"])
 def test_decode_append_head_major_placement_of_the_reference_classes(variant):
     """ref_rms.py:80-81 views the head-major product [H,M,D] as [M,H*D] without transposing back; with

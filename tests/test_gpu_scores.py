@@ -269,7 +269,9 @@ def test_fused_statistics_argument_rules():
 @pytest.mark.gpu
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,with_noise", [
     (1, 4, 4, 16, 1040, 128, False, True), (1, 4, 2, 16, 1040, 128, True, False), (2, 6, 1, 7, 332, 64, True, True),
-    (1, 71, 1, 16, 1040, 64, False, False), (1, 3, 3, 32, 36, 128, True, True), (1, 2, 2, 1, 100, 64, False, True)])
+    (1, 71, 1, 16, 1040, 64, False, False), (1, 3, 3, 32, 36, 128, True, True), (1, 2, 2, 1, 100, 64, False, True),
+    # odd key counts: the last row's last key sits in a dword that is half padding
+    (1, 4, 4, 16, 333, 128, True, True), (1, 2, 1, 16, 1041, 64, False, True), (1, 2, 2, 3, 35, 128, False, True)])
 def test_fused_statistics_with_fp16_noise_and_outputs(B, Hq, Hkv, Sq, Skv, D, causal, with_noise):
     """Held to the fp32 form of the same call bit for bit: the fp16 noise widened is the same noise, and an fp16 statistic
     is the fp32 one rounded once.  (The fp32 form is held to the oracle above.)"""

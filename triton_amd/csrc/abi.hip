@@ -2,7 +2,7 @@
 #include "attn.h"
 #include <string.h>
 
-extern "C" int trn_version(void) { return 100; }  // 0.1.0
+extern "C" int trn_version(void) { return 300; }  // 0.3.0: minor number = count of ABI revisions (entry points added)
 
 extern "C" const char* trn_status_name(int status) {
     switch (status) {

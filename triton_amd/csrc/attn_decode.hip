@@ -120,7 +120,10 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     constexpr int nsz = N16 ? 2 : 4;     // bytes per noise element
     const __amdgpu_buffer_rsrc_t nrs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(NOISE ? reinterpret_cast<const char*>(a.noise) + (b * a.nb + head * a.nh) * nsz : nullptr), 0,
-        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + a.Skv) * nsz) : 0, 0x00020000);
+        NOISE ? (int)(((int64_t)(a.Sq - 1) * a.ns + (N16 ? (a.Skv + 1) & ~1 : a.Skv)) * nsz) : 0, 0x00020000);
+    // (The range check works on whole dwords: with fp16 noise and an odd key count the last row's last key shares its
+    // dword with the first half of the row's padding, so the range ends behind that dword -- the rows are padded to
+    // 8 bytes -- and keys past the end are discarded by the mask, whatever the padding holds.)
     const int nvo = NOISE ? (int)(((int64_t)qrow_ld * a.ns + 4 * h) * nsz) : 0;
     float4_t g0[4], g1[4];
     auto fetch_noise = [&](int blk, float4_t (&g)[4]) __attribute__((always_inline)) {

@@ -108,6 +108,23 @@ def _row_stat(t: Optional[torch.Tensor], name: str, shape) -> None:
     _need(tuple(t.shape) == tuple(shape) and t.is_contiguous(), f"{name}: expected contiguous float32 {tuple(shape)}")
 
 
+_scratch_ready = set()
+
+
+def _static_scratch_ready(device: torch.device) -> None:
+    """The library looks up the address of its static scratch array once per GPU, which is no stream operation and
+    must not happen under graph capture: do it on the first eager "static" call on a device (trn_check_device), and
+    refuse a first call that arrives while the stream is capturing."""
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    if idx in _scratch_ready:
+        return
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError('workspace="static": make one eager call on this GPU (or call trn_check_device) before capturing')
+    with torch.cuda.device(idx):
+        _lib.check("trn_check_device", _lib.load().trn_check_device())
+    _scratch_ready.add(idx)
+
+
 def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor] = None,
               q_norm: bool = False, gamma_q: Optional[torch.Tensor] = None, q_eps: float = 0.0,
               noise: Optional[torch.Tensor] = None, tau: float = 1.0,
@@ -127,6 +144,7 @@ def attention(q, k, v, o, scale: float, causal: bool, lse: Optional[torch.Tensor
     lib = _lib.load()
     if isinstance(workspace, str):
         _need(workspace == "static", 'workspace: a uint8 GPU tensor, None, or "static"')
+        _static_scratch_ready(q.device)
         st = lib.trn_attn_fwd_noalloc_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(gamma_q),
                                           _ptr(noise), _ptr(lse_pert), _stream(q))
         _lib.check("trn_attn_fwd_noalloc_f16", st)
