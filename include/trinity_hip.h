@@ -189,6 +189,27 @@ int trn_attn_fwd_stats_f16(const trn_attn_desc* desc, const void* q, const void*
                            float* out_sum, float* out_sumsq, void* stream);
 
 /*
+ * trn_attn_fwd_stats_f16 with a workspace, for few queries and few heads on a LONG cache: the reference's KeyFormer
+ * and RoCo classes take any prefix length P (ref_rms.py:147-179, 249-280), and one workgroup per head sweeping tens
+ * of thousands of keys leaves most of the chip idle.  trn_attn_stats_workspace_bytes(desc) says for which problems
+ * the library would rather split (at most 32 queries per head, at most 48 heads in all, 8192 keys or more -- 4096
+ * with at most 16 heads) and how many bytes that takes, 0 otherwise.  Given a zero-initialised workspace of at least
+ * that many bytes (256-byte aligned, as for trn_attn_fwd_ws_f16) the attention runs with its keys split over
+ * workgroups, and the statistics -- which need the merged row normalisers -- follow as a second launch over all keys
+ * at once; lse (lse_pert with noise) is then required as the buffer that carries the normalisers between the two.
+ * Without a workspace, with one that is too small, without that buffer, or for a problem that would not be split,
+ * the call is trn_attn_fwd_stats_f16.  Results as trn_attn_fwd_stats_f16 to the stated tolerances (the shares are
+ * merged in a fixed order: the result does not depend on the run).  Neither has a counterpart in the reference, whose
+ * generated kernels load the whole key axis in one tile (TritonGen.py:2474-2547).
+ */
+int64_t trn_attn_stats_workspace_bytes(const trn_attn_desc* desc);
+int trn_attn_fwd_stats_ws_f16(const trn_attn_desc* desc, const void* q, const void* k, const void* v,
+                              void* o, float* lse, const void* gamma_q,
+                              const float* noise, float* lse_pert,
+                              float* out_sum, float* out_sumsq,
+                              void* workspace, int64_t workspace_bytes, void* stream);
+
+/*
  * trn_attn_fwd_stats_f16 with the noise and the statistics in fp16, for the reference's decode-append problem
  * (seq_q <= 32; TRN_E_UNSUPPORTED otherwise): its drivers allocate every tensor as fp16 -- C_out, C_out1, C_out2
  * (vanilla_llama_benchmark.py:131-139) and the noise (convert_eval_rms.py:201) -- and this entry point takes them as
@@ -265,7 +286,10 @@ int trn_gate_f16(const void* c1, const void* c2, void* out, int64_t rows, int64_
  * Measurement aid, no counterpart in the reference: the name (as a profiler's kernel trace prints it) of the kernel
  * instantiation that trn_attn_fwd_f16 launches for this problem -- decided by the same rules as the launch itself,
  * so that a benchmark can say which kernel its timing belongs to.  with_noise: as if a noise tensor were passed.
- * Returns "" for an invalid descriptor.  The string is static.
+ * It speaks for trn_attn_fwd_f16 only: fp32 noise, no workspace.  With at most 32 queries per head the other entry
+ * points launch the same kernel template with other last arguments -- fp16 noise (trn_attn_fwd_stats_half_f16) shows
+ * as <..., 2> where this function says <..., 1>, and a workspace that splits the keys turns the column shares
+ * (the middle argument) back to 1.  Returns "" for an invalid descriptor.  The string is static.
  */
 const char* trn_attn_fwd_kernel_name(const trn_attn_desc* desc, int32_t with_noise);
 

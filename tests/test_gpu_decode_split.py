@@ -176,3 +176,74 @@ def test_decode_modules_split_path_matches_reference_classes():
             close(t["O2"], ref.flatten_token_major(wo))
             # (q, k come from an fp16-rounded GEMM whose summation order differs from the oracle's: 5e-3 relative)
             close(t["C_out1"], s1, atol=1e-6, rtol=5e-3); close(t["C_out2"], s2, atol=1e-8, rtol=5e-3)
+
+
+# ---- trn_attn_fwd_stats_ws_f16: few heads on a long cache, keys split over workgroups, the statistics as a second launch
+STATS_SPLIT_CASES = [
+    # B, Hq, Hkv, Sq, Skv, D, causal, with_noise
+    (1, 8, 8, 16, 4112, 128, True, False), (1, 8, 2, 16, 4112, 128, False, True), (1, 16, 4, 5, 8200, 64, True, True),
+    (1, 32, 8, 16, 8208, 128, True, False), (2, 3, 3, 32, 4099, 128, False, True), (1, 12, 12, 1, 9000, 64, True, False)]
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,with_noise", STATS_SPLIT_CASES)
+def test_statistics_with_split_keys_match_oracle_and_single_launch(B, Hq, Hkv, Sq, Skv, D, causal, with_noise):
+    """RoCo's sums / KeyFormer's key scores over a long cache: the oracle at 1e-3 relative, and the single-launch form
+    of the same call (whose second sweep runs inside the attention kernel) to a tenth of that."""
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=23)
+    scale, tau = D ** -0.5, 1.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    n = ops.attention_stats_workspace_bytes(qd, kd, vd, torch.zeros_like(qd), scale, causal)
+    assert n > 0 and n == ops.attention_workspace_bytes(qd, kd, vd, torch.zeros_like(qd), scale, causal)
+    ws = torch.zeros(n, dtype=torch.uint8, device="cuda")
+    pitch = (Skv + 3) // 4 * 4
+    noise = None
+    if with_noise:
+        buf = torch.full((B, Hq, Sq, pitch), float("nan"))
+        buf[..., :Skv] = torch.randn(B, Hq, Sq, Skv, generator=torch.Generator().manual_seed(3))
+        noise = buf.cuda()[..., :Skv]
+    outs = []
+    for w in (ws, None):
+        o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda"); lsep = torch.zeros_like(lse)
+        s1 = torch.full((B, Hq, Skv), -1.0, device="cuda"); s2 = torch.full((B, Hq, Skv), -1.0, device="cuda")
+        kw = dict(noise=noise, tau=tau, lse_pert=lsep) if with_noise else {}
+        for _ in range(2):          # twice: the second call finds what the first left in the workspace
+            ops.attention_with_stats(qd, kd, vd, o, scale, causal, s1, None if with_noise else s2, lse=lse, workspace=w, **kw)
+        torch.cuda.synchronize()
+        outs.append((o, s1, s2, lse, lsep))
+    (o, s1, s2, lse, lsep), (o1, t1, t2, _, _) = outs
+    if with_noise:
+        wo, wscore = ref.keyformer(q, k, v, noise.cpu(), scale, tau, causal)
+        err = (s1.cpu() - wscore).abs()
+        assert (err <= 1e-9 + 1e-3 * wscore.abs()).all()
+    else:
+        wo, w1, w2 = ref.roco(q, k, v, scale, causal)
+        assert ((s1.cpu() - w1).abs() <= 1e-9 + 1e-3 * w1.abs()).all() and ((s2.cpu() - w2).abs() <= 1e-9 + 1e-3 * w2.abs()).all()
+        close(s2, t2, atol=1e-12, rtol=2e-4)
+    close(o, wo); close(o, o1, atol=2e-3, rtol=2e-3)
+    close(s1, t1, atol=1e-12, rtol=1e-4)
+
+
+def test_statistics_workspace_rule_and_fallbacks():
+    """Many heads fill the chip by themselves, short caches are launch-bound: no split there, and the entry point with
+    a workspace is then the plain one bit for bit; so it is with a workspace that is too small or without the buffer
+    for the row normalisers."""
+    from triton_amd import ops
+    scale = 0.125
+    for (B, Hq, Hkv, Sq, Skv, D), want_split in (((1, 71, 1, 16, 16400, 64), False), ((1, 32, 8, 16, 4112, 128), False),
+                                                  ((1, 8, 8, 16, 2064, 128), False), ((1, 8, 8, 33, 8208, 128), False),
+                                                  ((1, 32, 8, 16, 8208, 128), True), ((1, 16, 16, 4, 4112, 64), True)):
+        q = torch.zeros(B, Hq, Sq, D, dtype=torch.float16, device="cuda"); k = torch.zeros(B, Hkv, Skv, D, dtype=torch.float16, device="cuda")
+        assert (ops.attention_stats_workspace_bytes(q, k, k, q, scale, True) > 0) == want_split, (Hq, Skv)
+    q, k, v = make(1, 8, 8, 16, 4112, 128, seed=29)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    n = ops.attention_stats_workspace_bytes(qd, kd, vd, qd, scale, True)
+    res = []
+    for ws, with_lse in ((None, True), (torch.zeros(n // 2 // 256 * 256, dtype=torch.uint8, device="cuda"), True),
+                         (torch.zeros(n, dtype=torch.uint8, device="cuda"), False)):
+        o = torch.zeros_like(qd); s1 = torch.zeros(1, 8, 4112, device="cuda"); lse = torch.zeros(1, 8, 16, device="cuda")
+        ops.attention_with_stats(qd, kd, vd, o, scale, True, s1, None, lse=lse if with_lse else None, workspace=ws)
+        torch.cuda.synchronize()
+        res.append((o, s1))
+    for o, s1 in res[1:]:
+        assert torch.equal(o, res[0][0]) and torch.equal(s1, res[0][1])

@@ -196,6 +196,31 @@ def test_decode_append_modules_match_reference_classes(amp, M, N, D, P):
     close(t["O2"], ref.flatten_token_major(wo), atol); close(t["C_out1"], s1, 1e-6, srt); close(t["C_out2"], s2, 1e-8, srt)
 
 
+@pytest.mark.parametrize("variant", ["keyformer", "roco"])
+def test_decode_score_modules_on_a_long_cache_split_their_keys(variant):
+    """Eight heads on a 4096-token cache: the modules take the library's split path (keys over workgroups, statistics as
+    a second launch) with the reference's fp16 tensors converted on the way; whole-module outputs against the oracle."""
+    from triton_amd import modules, ops
+    M, N, D, P = 16, 1024, 128, 4096
+    cpu, H = _decode_tensors(M, N, D, P, seed=9)
+    W = (cpu["WQ"], cpu["WK"], cpu["WV"])
+    t = {k: v.cuda() for k, v in cpu.items()}
+    t["O2"] = torch.zeros(M, N, dtype=torch.float16, device="cuda")
+    t["C_out"] = torch.zeros(H, P + M, dtype=torch.float16, device="cuda")
+    t["C_out1"] = torch.zeros(H, P + M, device="cuda"); t["C_out2"] = torch.zeros(H, P + M, device="cuda")
+    qv = torch.zeros(1, H, M, D, dtype=torch.float16, device="cuda")
+    assert ops.attention_stats_workspace_bytes(qv, t["K_cache"][None], t["V_cache"][None], qv, 1.0, False) > 0
+    m = modules.get(variant, "decode", head_dim=D)
+    drive(m, t, ["O2", "C_out", "C_out1", "C_out2"])
+    if variant == "keyformer":
+        wo, pw = ref.decode_append_keyformer(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], cpu["noise"], P, D, tau=1.5)
+        close(t["C_out"], pw.sum(dim=1), 1e-4, 2e-3)
+    else:
+        wo, s1, s2 = ref.decode_append_roco(cpu["X"], *W, cpu["K_cache"], cpu["V_cache"], P, D)
+        close(t["C_out1"], s1, 1e-6, 1e-3); close(t["C_out2"], s2, 1e-8, 1e-3)
+    close(t["O2"], ref.flatten_token_major(wo), 1e-4)
+
+
 @pytest.mark.parametrize("variant", ["vanilla", "keyformer", "roco"])
 def test_decode_modules_driven_the_old_way_eagerly_with_block_keywords(variant):
     """The older drivers' call shape (rms_benchmark.py:247-265): no graph, every call eager on the current stream,

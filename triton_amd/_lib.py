@@ -18,7 +18,7 @@ EXPORTS = (
     "trn_attn_fwd_f16", "trn_attn_colstats_f16", "trn_prenorm_qkv_f16", "trn_calibration_copy",
     "trn_calibration_mfma", "trn_attn_workspace_bytes", "trn_attn_fwd_ws_f16", "trn_linear_f16", "trn_gate_f16", "trn_attn_fwd_stats_f16",
     "trn_attn_fwd_noalloc_f16", "trn_attn_fwd_kernel_name", "trn_attn_colmeanstd_f16", "trn_attn_fwd_probs_f16",
-    "trn_attn_fwd_stats_half_f16",
+    "trn_attn_fwd_stats_half_f16", "trn_attn_fwd_stats_ws_f16", "trn_attn_stats_workspace_bytes",
 )
 
 
@@ -73,6 +73,10 @@ def load() -> C.CDLL:
     lib.trn_attn_fwd_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.trn_attn_fwd_stats_f16.restype = C.c_int
     lib.trn_attn_fwd_stats_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
+    lib.trn_attn_stats_workspace_bytes.restype = C.c_int64
+    lib.trn_attn_stats_workspace_bytes.argtypes = [C.POINTER(AttnDesc)]
+    lib.trn_attn_fwd_stats_ws_f16.restype = C.c_int
+    lib.trn_attn_fwd_stats_ws_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, i64, vp]
     lib.trn_attn_fwd_stats_half_f16.restype = C.c_int
     lib.trn_attn_fwd_stats_half_f16.argtypes = [C.POINTER(AttnDesc), vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp]
     lib.trn_linear_f16.restype = C.c_int

@@ -476,6 +476,40 @@ extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, con
     return trn_attn_colstats_f16(d, q, k, rows, noise, out_sum, out_sumsq, stream);
 }
 
+// Where two launches (keys split over workgroups, then the statistics over all keys at once) beat the single launch
+// whose statistics sweep runs with one workgroup per head and column share.  Measured, 16 queries per head, microseconds
+// one launch / two launches: 8 heads of 128: 43 / 35 at 4 k keys, 156 / 52 at 16 k; 16 heads of 64: 30 / 30 at 4 k,
+// 55 / 41 at 8 k; 32 heads of 128: 45 / 52 at 4 k, 82 / 77 at 8 k, 169 / 130 at 16 k; 71 heads of 64: 33 / 60 at 4 k,
+// 126 / 182 at 16 k (that many heads fill the chip by themselves).
+extern "C" int64_t trn_attn_stats_workspace_bytes(const trn_attn_desc* d) {
+    const int64_t need = trn_attn_workspace_bytes(d);
+    if (need == 0) return 0;
+    const int64_t n_bh = (int64_t)d->batch * d->n_q_heads;
+    return n_bh <= 48 && d->seq_kv >= (n_bh <= 16 ? 4096 : 8192) ? need : 0;
+}
+
+extern "C" int trn_attn_fwd_stats_ws_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
+                                         float* lse, const void* gamma_q, const float* noise, float* lse_pert,
+                                         float* out_sum, float* out_sumsq, void* workspace, int64_t workspace_bytes,
+                                         void* stream) {
+    using namespace trn;
+    if (!d) return TRN_E_NULL;
+    if (!out_sum && !out_sumsq) return TRN_E_NULL;
+    if (d->q_norm) return TRN_E_UNSUPPORTED;
+    if (workspace && ((reinterpret_cast<uintptr_t>(workspace) & 255u) != 0 || workspace_bytes < 0)) return TRN_E_ALIGN;
+    // Few queries and few heads on a long cache: the keys are split over workgroups (which needs the workspace), and
+    // the statistics, which need the merged row normalisers, follow as a launch of their own over all keys at once --
+    // if the caller gave the buffer that carries the normalisers.  Everything else runs as trn_attn_fwd_stats_f16.
+    const int64_t need = trn_attn_stats_workspace_bytes(d);
+    float* rows = noise ? lse_pert : lse;
+    if (workspace && need > 0 && workspace_bytes >= need && rows) {
+        const int st = attn_forward(d, q, k, v, o, lse, gamma_q, noise, lse_pert, workspace, workspace_bytes, nullptr, nullptr, stream);
+        if (st != TRN_OK) return st;
+        return trn_attn_colstats_f16(d, q, k, rows, noise, out_sum, out_sumsq, stream);
+    }
+    return trn_attn_fwd_stats_f16(d, q, k, v, o, lse, gamma_q, noise, lse_pert, out_sum, out_sumsq, stream);
+}
+
 extern "C" int trn_attn_fwd_stats_half_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
                                            float* lse, const void* gamma_q, const void* noise, float* lse_pert,
                                            void* out_sum, void* out_sumsq, void* stream) {

@@ -300,14 +300,20 @@ class _DecodeAppend(FusedModule):
         H, M, D = q.shape
         o = self._o_view(O2, H, M, D)
         nbytes = ops.attention_workspace_bytes(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal)
-        ws = None
-        if nbytes:
-            key = ("attn_ws", (nbytes,), torch.uint8, str(q.device))
-            fresh = key not in self._ws
-            ws = self._workspace("attn_ws", (nbytes,), torch.uint8, q.device)
-            if fresh:
-                ws.zero_()
-        ops.attention(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal, workspace=ws, **kw)
+        ops.attention(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
+                      workspace=self._split_ws(nbytes, q.device), **kw)
+
+    def _split_ws(self, nbytes: int, device):
+        """The split-key workspace (zeroed once, on the cold call that allocates it; the kernels leave its counters at
+        zero), or None when the library would not split this problem."""
+        if not nbytes:
+            return None
+        key = ("attn_ws", (nbytes,), torch.uint8, str(device))
+        fresh = key not in self._ws
+        ws = self._workspace("attn_ws", (nbytes,), torch.uint8, device)
+        if fresh:
+            ws.zero_()
+        return ws
 
 
 class DecodeVanilla(_DecodeAppend):
@@ -346,7 +352,11 @@ class DecodeKeyFormer(_DecodeAppend):
         H, M, D = q.shape
         PM = K_cache.shape[1]
         lsep = self._workspace("lse_pert", (1, H, M), torch.float32, X.device)
-        if self.reduce and M <= 32 and _half_io_ok(C_out, (H, PM)) and _half_noise_ok(noise):
+        o = self._o_view(O2, H, M, D)
+        # few heads on a long cache: keys split over workgroups, the key scores as a second launch (fp32 on the way)
+        split = ops.attention_stats_workspace_bytes(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal) \
+            if self.reduce else 0
+        if not split and self.reduce and M <= 32 and _half_io_ok(C_out, (H, PM)) and _half_noise_ok(noise):
             # everything fp16 as the reference's drivers allocate it: one launch, no copies on the side
             ops.attention_with_stats_half(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale,
                                           self.causal, C_out.view(1, H, PM), None, noise=noise[None], tau=self.tau,
@@ -358,11 +368,11 @@ class DecodeKeyFormer(_DecodeAppend):
             raise ValueError(f"C_out {tuple(C_out.shape)}: expected {shape[1:]}")
         score = C_out.view(shape) if C_out.dtype == torch.float32 and C_out.is_contiguous() else \
             self._workspace("score32", shape, torch.float32, X.device)
-        o = self._o_view(O2, H, M, D)
         if self.reduce:
             # one launch up to 32 new tokens (the key scores are a second sweep inside the attention kernel), two beyond
             ops.attention_with_stats(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
-                                     score, None, noise=n4, tau=self.tau, lse_pert=lsep)
+                                     score, None, noise=n4, tau=self.tau, lse_pert=lsep,
+                                     workspace=self._split_ws(split, X.device))
         else:
             ops.attention_with_probs(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
                                      score, noise=n4, tau=self.tau, lse_pert=lsep)
@@ -378,16 +388,19 @@ class DecodeRoCo(_DecodeAppend):
         H, M, D = q.shape
         PM = K_cache.shape[1]
         lse = self._workspace("lse", (1, H, M), torch.float32, X.device)
-        if M <= 32 and _half_io_ok(C_out1, (H, PM)) and _half_io_ok(C_out2, (H, PM)):
-            ops.attention_with_stats_half(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale,
+        o = self._o_view(O2, H, M, D)
+        # few heads on a long cache: keys split over workgroups, the statistics as a second launch (fp32 on the way)
+        split = ops.attention_stats_workspace_bytes(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal)
+        if not split and M <= 32 and _half_io_ok(C_out1, (H, PM)) and _half_io_ok(C_out2, (H, PM)):
+            ops.attention_with_stats_half(q[None], K_cache[None], V_cache[None], o, self.scale,
                                           self.causal, C_out1.view(1, H, PM), C_out2.view(1, H, PM), lse=lse)
             return
         outs = []
         for i, c in enumerate((C_out1, C_out2)):
             outs.append(c.view(1, H, PM) if c.dtype == torch.float32 and c.is_contiguous() else
                         self._workspace(f"stat32_{i}", (1, H, PM), torch.float32, X.device))
-        ops.attention_with_stats(q[None], K_cache[None], V_cache[None], self._o_view(O2, H, M, D), self.scale, self.causal,
-                                 outs[0], outs[1], lse=lse)
+        ops.attention_with_stats(q[None], K_cache[None], V_cache[None], o, self.scale, self.causal,
+                                 outs[0], outs[1], lse=lse, workspace=self._split_ws(split, X.device))
         _store_scores(C_out1, outs[0]); _store_scores(C_out2, outs[1])
 
 

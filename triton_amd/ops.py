@@ -172,6 +172,13 @@ def attention_workspace_bytes(q, k, v, o, scale: float, causal: bool) -> int:
     return int(_lib.load().trn_attn_workspace_bytes(C.byref(d)))
 
 
+def attention_stats_workspace_bytes(q, k, v, o, scale: float, causal: bool) -> int:
+    """Bytes of workspace with which `attention_with_stats` would split the keys of this problem over several
+    workgroups and run the statistics as a second launch (0: it would not -- one launch is faster)."""
+    d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, None, 1.0)
+    return int(_lib.load().trn_attn_stats_workspace_bytes(C.byref(d)))
+
+
 def attention_colstats(q, k, lse, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
                        out_sumsq: Optional[torch.Tensor] = None, noise: Optional[torch.Tensor] = None,
                        tau: float = 1.0) -> None:
@@ -225,10 +232,13 @@ def attention_col_mean_std(q, k, lse, scale: float, causal: bool, out_mean: torc
 def attention_with_stats(q, k, v, o, scale: float, causal: bool, out_sum: Optional[torch.Tensor],
                          out_sumsq: Optional[torch.Tensor] = None, lse: Optional[torch.Tensor] = None,
                          noise: Optional[torch.Tensor] = None, tau: float = 1.0,
-                         lse_pert: Optional[torch.Tensor] = None) -> None:
+                         lse_pert: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None) -> None:
     """`attention` and `attention_colstats` in one call (one launch with at most 32 queries per head): o, and the
     column sums / sums of squares of the probabilities -- of the perturbed ones when noise is given.  With more than
-    32 queries lse (lse_pert with noise) must be given: it carries the row normalisers between the two kernels."""
+    32 queries lse (lse_pert with noise) must be given: it carries the row normalisers between the two kernels.
+    workspace: optional zero-initialised uint8 tensor of attention_workspace_bytes(...) bytes: few queries on a long
+    cache then run with their keys split over workgroups and the statistics as a second launch (lse / lse_pert
+    required, as above)."""
     d = _attn_desc(q, k, v, o, scale, causal, False, 0.0, noise, tau)
     B, Hq, Sq, _ = q.shape
     Skv = k.shape[2]
@@ -238,6 +248,13 @@ def attention_with_stats(q, k, v, o, scale: float, causal: bool, out_sum: Option
     if noise is not None:
         _need(lse_pert is not None, "noise requires lse_pert")
     lib = _lib.load()
+    if workspace is not None:
+        _need(workspace.is_cuda and workspace.is_contiguous() and workspace.dtype == torch.uint8, "workspace: expected a contiguous uint8 GPU tensor")
+        st = lib.trn_attn_fwd_stats_ws_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), None, _ptr(noise),
+                                           _ptr(lse_pert), _ptr(out_sum), _ptr(out_sumsq), _ptr(workspace), workspace.numel(),
+                                           _stream(q))
+        _lib.check("trn_attn_fwd_stats_ws_f16", st)
+        return
     st = lib.trn_attn_fwd_stats_f16(C.byref(d), _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), None, _ptr(noise),
                                     _ptr(lse_pert), _ptr(out_sum), _ptr(out_sumsq), _stream(q))
     _lib.check("trn_attn_fwd_stats_f16", st)
