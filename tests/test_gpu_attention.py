@@ -107,6 +107,32 @@ def test_attention_parity_seeded_random_shapes(B, Hq, Hkv, Sq, Skv, D, causal, q
     close(lse, want_lse, atol=1e-3, rtol=1e-3)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal", [
+    (1, 4, 2, 300, 300, 128, True), (1, 4, 4, 256, 520, 64, False), (2, 32, 8, 1024, 1024, 128, True),
+    (1, 32, 8, 2048, 2048, 128, True), (1, 8, 1, 700, 700, 64, True), (1, 4, 2, 16, 1040, 128, True)])
+def test_attention_scores_that_rise_and_jump_along_the_keys(B, Hq, Hkv, Sq, Skv, D, causal):
+    """The kernels keep a lazy reference maximum, set by the first 32-key block and raised only when a later block
+    exceeds it by more than 2^8; N(0,1) inputs never get there.  Here the keys grow sevenfold along the sequence, so the
+    block maxima climb through several raises, and three late keys are multiples of particular queries, so that single
+    scores jump tens of binades above everything before them (a probability formed against the old reference would be
+    infinite in fp16).  Outputs and row normalisers against the oracle at the usual tolerances."""
+    from triton_amd import ops
+    q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=31)
+    k = (k.float() * (1.0 + 6.0 * torch.arange(Skv).float() / Skv)[None, None, :, None]).half()
+    G = Hq // Hkv
+    for key, qi in ((Skv - 3, Sq - 1), (Skv // 2 + 5, Sq // 2), (40, min(Sq - 1, 45))):     # key j = 3 x query qi of the KV head's first query head
+        k[:, :, key] = (3.0 * q[:, ::G, qi].float()).half()
+    scale = D ** -0.5
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    o = torch.zeros_like(qd); lse = torch.zeros(B, Hq, Sq, device="cuda")
+    ops.attention(qd, kd, vd, o, scale, causal, lse=lse)
+    torch.cuda.synchronize()
+    want, want_lse = ref.attention(q, k, v, scale, causal, return_lse=True)
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    close(o, want)
+    close(lse, want_lse, atol=2e-3, rtol=1e-3)
+
+
 def test_attention_reference_recipe_unscaled():
     """The reference's own input recipe and semantics: scale 1, no mask (ref_rms.py:77-78)."""
     from triton_amd import ops
