@@ -379,12 +379,20 @@ def main():
     # HBM bytes per launch of the dominant kernel, measured offline with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
     # (recipe and scaling in profiles/); null until that file exists.
     traffic = None
+    traffic_of = None       # SHA-256 of the kernel source the counters were taken on
     tpath = os.path.join(ROOT, "profiles", "attn_fwd_llama3_s4096_hbm_traffic.txt")
     if os.path.exists(tpath):
         with open(tpath) as f:
             for ln in f:
                 if ln.startswith("hbm_bytes_per_launch:"):
                     traffic = int(ln.split(":")[1])
+                if ln.startswith("kernel_source_sha256:"):
+                    traffic_of = ln.split(":")[1].strip()
+    import hashlib
+    with open(os.path.join(ROOT, "triton_amd", "csrc", "attn_fwd16.hip"), "rb") as f:
+        src_now = hashlib.sha256(f.read()).hexdigest()
+    # (the figure is a counter reading taken offline: say so when the kernel's source has changed since)
+    traffic_current = traffic is not None and traffic_of == src_now
     line = {
         "metric": "attn TFLOP/s + % fp16 MFMA peak (Llama3-8B, S=4096); RMSNorm HBM GB/s",
         "value": round(van["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -400,7 +408,8 @@ def main():
                      "kernel": van["kernel"], "kernel_ms": round(van["kernel_ms"], 5),
                      "kernel_ms_per_region": [round(x, 5) for x in van["region_ms"]],
                      "traffic_source": "profiles/attn_fwd_llama3_s4096_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / "
-                                       "WRITE_SIZE of this command, scaled by the library's copy kernel)"},
+                                       "WRITE_SIZE of this command, scaled by the library's copy kernel)",
+                     "traffic_taken_on_this_kernel_source": traffic_current},
     }
     ceil = mfma_ceiling()
     line["roofline"]["mfma_only_kernel_tflops"] = {k: round(v, 1) for k, v in ceil.items()}
