@@ -172,6 +172,26 @@ def test_no_workspace_exceeds_the_static_scratch_array(lib):
     assert 0 < largest <= capacity, (largest, capacity)
 
 
+def test_statistics_split_rule_on_the_host(lib):
+    """trn_attn_stats_workspace_bytes: the long-cache rule (few heads, many keys, at most 32 queries per head) is host
+    arithmetic; where it says split, the size is that of the attention's own split workspace."""
+    def need(heads, sq, skv, D=128, fn=lib.trn_attn_stats_workspace_bytes):
+        d = _desc(batch=1, n_q_heads=heads, n_kv_heads=1, seq_q=sq, seq_kv=skv, head_dim=D, causal=0,
+                  q_stride_b=heads * sq * D, q_stride_h=sq * D, q_stride_s=D, k_stride_b=skv * D, k_stride_h=skv * D,
+                  k_stride_s=D, v_stride_b=skv * D, v_stride_h=skv * D, v_stride_s=D, o_stride_b=heads * sq * D,
+                  o_stride_h=sq * D, o_stride_s=D)
+        return fn(C.byref(d))
+    for heads, sq, skv, D, split in ((8, 16, 4096, 128, True), (8, 16, 4000, 128, False), (16, 16, 4096, 64, True),
+                                     (17, 16, 4096, 128, False), (32, 16, 8192, 128, True), (32, 16, 8191, 128, False),
+                                     (48, 4, 16384, 128, True), (49, 4, 16384, 128, False), (71, 16, 65536, 64, False),
+                                     (8, 33, 16384, 128, False), (8, 1, 1040, 128, False)):
+        got = need(heads, sq, skv, D)
+        assert (got > 0) == split, (heads, sq, skv, D, got)
+        if split:
+            assert got == need(heads, sq, skv, D, lib.trn_attn_workspace_bytes)
+    assert lib.trn_attn_stats_workspace_bytes(None) == 0
+
+
 def test_a_missing_library_is_an_error_not_a_fallback(monkeypatch, tmp_path):
     from triton_amd import _lib
     monkeypatch.setattr(_lib, "_lib", None)
