@@ -11,9 +11,10 @@
 //     NB consecutive groups and may straddle two outputs: every group has its own buffer descriptor, and every
 //     32-column block of the epilogue its own output.
 //   * Both operands go straight from global memory into LDS (buffer_load ... lds, XOR-swizzled rows); no
-//     register staging and no LDS writes from the VALU.  gamma is multiplied into the X operand after it is read
-//     back from LDS (one packed fp16 multiply per pair: the correctly rounded product), and the waves of the
-//     first column group also sum its squares with the fp32 dot-product instruction for the row rstd.
+//     register staging and no LDS writes from the VALU.  gamma is multiplied into the W operand after it is read
+//     back from LDS (one packed fp16 multiply per pair: the correctly rounded product; a lane's W^T operand holds the
+//     same eight contraction columns as its X^T operand, and a step has NB W operands against four X operands), and
+//     the waves of the first column group sum the squares of X with the fp32 dot-product instruction for the row rstd.
 //   * Four stages of 32 contraction columns: a stage is requested three k-tiles before its first use,
 //     which at 256 x 256 flops per staged column covers the L2 / HBM latency.
 //   * The one barrier per k-tile sits between the two 16-column halves of the tile's MFMAs, after the second
@@ -30,7 +31,7 @@ namespace trn {
 // x four consecutive chunks of one phase of the transposing read touch every bank once.
 __device__ __forceinline__ int gswz(int r) { return (((r >> 1) & 1) << 2) | ((r >> 2) & 3); }
 
-// G: gamma is multiplied into the X operand (norm on and a gamma given); without it the multiply, the gamma
+// G: gamma is multiplied into the W operand (norm on and a gamma given); without it the multiply, the gamma
 // loads and their ring leave the loop.
 template <int NB, bool G>
 __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs a) {
@@ -105,7 +106,8 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     } while (0)
 #define TRN_FETCH(kt_, xd_, wd_) _Pragma("unroll") for (int fi_ = 0; fi_ < 4; ++fi_) TRN_FETCH_ONE(kt_, xd_, wd_, fi_)
 
-    // ---- gamma: the X^T operand of contraction step ks holds columns kt*32 + ks*16 + 8h .. +7 of its token.
+    // ---- gamma: the operands of contraction step ks hold columns kt*32 + ks*16 + 8h .. +7 (of the lane's token in
+    // X^T, of the lane's output column in W^T).
     constexpr bool use_g = G;
     const bool stats = a.norm && wn == 0;
     const __amdgpu_buffer_rsrc_t grs = __builtin_amdgcn_make_buffer_rsrc(
@@ -157,20 +159,23 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     float ss[4] = {0.f, 0.f, 0.f, 0.f};
     // One contraction step = 4 groups (one token block each) of NB MFMAs.  A wave has its SIMD to itself, so
     // whatever else it issues must sit between MFMAs or the pipe runs dry: every MFMA heads a slot that also
-    // carries a piece of the other work -- the sum of squares and gamma multiply of the NEXT group's operand
-    // (the next step's first one in the last group), the next step's operand reads (W operands first: its first
-    // group needs all of them), and, in the second step of a k-tile, a quarter of the stage refill.
+    // carries a piece of the other work -- the sum of squares of the NEXT group's X operand (the next step's first
+    // one in the last group), the next step's operand reads (W operands first: its first group needs all of them),
+    // the gamma multiply of those W operands in the last group (by then they have arrived), and, in the second step
+    // of a k-tile, a quarter of the stage refill.
     auto step = [&](half8_t& xv, half8_t (&xb)[4], half8_t (&wa)[NB], const half8_t& g, half8_t (&xn)[4],
                     half8_t (&wn_)[NB], const half_t* Xr, const half_t* Wr, int ks_r, const half8_t& gn,
                     auto&& extra) __attribute__((always_inline)) {
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
-            acc[0][mb] = mfma32(wa[0], xv, acc[0][mb]);
+            // (the column blocks are walked forwards for even token blocks and backwards for odd ones, so that from one MFMA
+            // to the next only one of the two operands changes: 0.5 % of the kernel's time at the board's power limit)
+            { constexpr int z = 0; const int nbx = (mb & 1) ? NB - 1 - z : z; acc[nbx][mb] = mfma32(wa[nbx], xv, acc[nbx][mb]); }
             if (mb == 0) wn_[0] = read_w(Wr, ks_r, 0);
             if (mb == 1) wn_[2] = read_w(Wr, ks_r, 2);
             if (mb >= 2) xn[mb] = read_x(Xr, ks_r, mb);
             __builtin_amdgcn_sched_barrier(0);
-            acc[1][mb] = mfma32(wa[1], xv, acc[1][mb]);
+            { constexpr int z = 1; const int nbx = (mb & 1) ? NB - 1 - z : z; acc[nbx][mb] = mfma32(wa[nbx], xv, acc[nbx][mb]); }
             const half8_t raw = mb < 3 ? xb[mb + 1] : xn[0];
             if (stats) {
 #pragma unroll
@@ -183,15 +188,21 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
                 if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
             }
             __builtin_amdgcn_sched_barrier(0);
-            acc[2][mb] = mfma32(wa[2], xv, acc[2][mb]);
-            const half8_t xv_next = G ? raw * (mb < 3 ? g : gn) : raw;
+            { constexpr int z = 2; const int nbx = (mb & 1) ? NB - 1 - z : z; acc[nbx][mb] = mfma32(wa[nbx], xv, acc[nbx][mb]); }
+            const half8_t xv_next = raw;
             if constexpr (NB == 4) {
                 if (mb == 0) wn_[1] = read_w(Wr, ks_r, 1);
                 if (mb == 1) wn_[3] = read_w(Wr, ks_r, 3);
                 __builtin_amdgcn_sched_barrier(0);
-                acc[3][mb] = mfma32(wa[3], xv, acc[3][mb]);
+                { constexpr int z = 3; const int nbx = (mb & 1) ? NB - 1 - z : z; acc[nbx][mb] = mfma32(wa[nbx], xv, acc[nbx][mb]); }
             }
             if (mb < 2) xn[mb] = read_x(Xr, ks_r, mb);
+            if constexpr (G) {
+                if (mb == 3) {
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) wn_[nb] = wn_[nb] * gn;
+                }
+            }
             extra(mb);
             __builtin_amdgcn_sched_barrier(0);
             xv = xv_next;
@@ -213,7 +224,7 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
     for (int i = 0; i < 4; ++i) xb0[i] = read_x(Xs0, 0, i);
 #pragma unroll
     for (int i = 0; i < NB; ++i) wa0[i] = read_w(Ws0, 0, i);
-    half8_t xv = xb0[0];                    // the operand of the next MFMA group, gamma applied
+    half8_t xv = xb0[0];                    // the X operand of the next MFMA group
     if (stats) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -221,7 +232,10 @@ __global__ __launch_bounds__(256, 1) void prenorm_qkv_wide_kernel(const GemmArgs
             ss[0] = __builtin_amdgcn_fdot2(p, p, ss[0], false);
         }
     }
-    if (G) xv = xv * g0[0];
+    if (G) {
+#pragma unroll
+        for (int i = 0; i < NB; ++i) wa0[i] = wa0[i] * g0[0];
+    }
 
     // k-tile kt reads stage kt%4: the operands of its first step during the second step of k-tile kt-1, those of
     // its second step during its first.  From the barrier between the two steps on, the stage is free and is
