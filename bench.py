@@ -41,6 +41,13 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="with --workload all: skip the decode-append timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
+    ap.add_argument("--inputs", default="randn", choices=("randn", "zeros"),
+                    help="zeros: run the headline attention on all-zero Q, K, V instead of the benchmark's N(0,1) data -- a "
+                         "diagnostic for profiler runs (same instructions, no switching activity: the difference is the "
+                         "board's clock under its power limit); the line's `data` says so and it is not the benchmark")
+    ap.add_argument("--no-zero-leg", action="store_true",
+                    help="skip the all-zero-input diagnostic launch of the headline kernel (profiler runs: every dispatch "
+                         "of the kernel in the trace is then the benchmark's)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run the library's plain copy kernel on 256 MiB (3 launches) so that a rocprofv3 --pmc run "
                          "of this command holds a kernel of known HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
@@ -154,18 +161,27 @@ def attn_inputs(cfg, seed=42):
     return q, k, v
 
 
-def bench_vanilla(steps, warmup):
+def bench_vanilla(steps, warmup, inputs="randn", zero_leg=True):
     import torch
     from triton_amd import configs, modules
     cfg = configs.VANILLA
     q, k, v = attn_inputs(cfg)
     t = dict(Q=q.cuda(), K=k.cuda(), V=v.cuda(), O=torch.zeros_like(q).cuda())
+    if inputs == "zeros":
+        for name in "QKV":
+            t[name].zero_()
     wall, ev, samples = graph_timed(modules.get("vanilla"), t, steps, warmup, with_samples=True)
+    zero_ms = None
+    if inputs == "randn" and zero_leg:
+        # The same launch on all-zero inputs (same instructions and memory traffic, no switching activity in the
+        # datapaths): what the kernel's cycles alone take when the board does not lower its clock.
+        tz = {name: torch.zeros_like(x) for name, x in t.items()}
+        _, zero_ms = graph_timed(modules.get("vanilla"), tz, min(steps, 100), warmup)
     flops = configs.attn_flops(cfg["batch"], cfg["n_heads"], cfg["seq"], cfg["seq"], cfg["head_dim"], True)
     from triton_amd import ops
     kernel = ops.attention_kernel_name(t["Q"], t["K"], t["V"], t["O"], cfg["head_dim"] ** -0.5, True)
     return dict(wall_ms=wall, kernel_ms=ev, flops=flops, tflops=flops / wall / 1e9, kernel_tflops=flops / ev / 1e9,
-                tensors=(q, k, v), kernel=kernel, region_ms=samples)
+                tensors=(q, k, v), kernel=kernel, region_ms=samples, zero_inputs_kernel_ms=zero_ms)
 
 
 def bench_rmsnorm(steps, warmup):
@@ -353,7 +369,7 @@ def main():
         del src, dst
     wl = a.workload
     extra = {}
-    van = bench_vanilla(a.steps, a.warmup) if wl in ("headline", "all", "vanilla") else None
+    van = bench_vanilla(a.steps, a.warmup, a.inputs, not a.no_zero_leg) if wl in ("headline", "all", "vanilla") else None
     if wl in ("headline", "all", "rmsnorm"):
         extra["rmsnorm"] = bench_rmsnorm(a.steps, a.warmup)
     def guarded(fn, *args):
@@ -397,7 +413,7 @@ def main():
         "metric": "attn TFLOP/s + % fp16 MFMA peak (Llama3-8B, S=4096); RMSNorm HBM GB/s",
         "value": round(van["tflops"], 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(van["wall_ms"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f16", "data": "synthetic",
+        "dtype": "f16", "data": "synthetic" if a.inputs == "randn" else "all-zero inputs: a diagnostic run, not the benchmark",
         "config": {"workload": "vanilla causal GQA attention, batch 1, seq 4096, 32 q heads / 8 kv heads, head_dim 128",
                    "flops_per_step": van["flops"], "flop_convention": "4*B*H*S^2*D/2 (causal-halved)",
                    "timing": f"graph replay on a side stream, 20 forwards per graph; {CLOCK_WARMUP_S} s of untimed replays, "
@@ -414,6 +430,11 @@ def main():
     ceil = mfma_ceiling()
     line["roofline"]["mfma_only_kernel_tflops"] = {k: round(v, 1) for k, v in ceil.items()}
     line["roofline"]["frac_of_mfma_only_random_operands"] = round(van["kernel_tflops"] / ceil["random_operands"], 4)
+    if van["zero_inputs_kernel_ms"] is not None:
+        line["roofline"]["same_kernel_on_all_zero_inputs"] = {
+            "kernel_ms": round(van["zero_inputs_kernel_ms"], 5),
+            "frac": round(van["flops"] / van["zero_inputs_kernel_ms"] / 1e9 / peak, 4),
+            "note": "diagnostic: same instructions and traffic without switching activity (the board holds its clock)"}
     if "rmsnorm" in extra:
         r = extra["rmsnorm"]
         line["rmsnorm"] = {"value": round(r["gbps"], 1), "unit": "GB/s", "frac_of_hbm_peak": round(r["frac"], 4),
