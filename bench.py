@@ -37,7 +37,7 @@ def parse():
     ap.add_argument("--workload", default="all",
                     help="all (the headline, RMSNorm, the four other prefill workloads and the decode-append timings: the "
                          "default), headline (vanilla attention + RMSNorm only), or one of vanilla rmsnorm prenorm qknorm "
-                         "keyformer roco decode")
+                         "keyformer roco decode, or sweep (vanilla attention over sequence lengths and head shapes)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="with --workload all: skip the decode-append timings")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget for the CPU baseline sample")
@@ -182,6 +182,37 @@ def bench_vanilla(steps, warmup, inputs="randn", zero_leg=True):
     kernel = ops.attention_kernel_name(t["Q"], t["K"], t["V"], t["O"], cfg["head_dim"] ** -0.5, True)
     return dict(wall_ms=wall, kernel_ms=ev, flops=flops, tflops=flops / wall / 1e9, kernel_tflops=flops / ev / 1e9,
                 tensors=(q, k, v), kernel=kernel, region_ms=samples, zero_inputs_kernel_ms=zero_ms)
+
+
+def bench_sweep(steps, warmup):
+    """Vanilla attention over sequence lengths and the two head shapes of the benchmark configurations (not part of the
+    default run): TFLOP/s on N(0,1) inputs and on all-zero inputs per shape, same timing method as the headline."""
+    import torch
+    from triton_amd import configs, modules
+    m = modules.get("vanilla")
+    rows = []
+    shapes = [("llama3 GQA 32/8 x 128", 1, 32, 8, 128, S, True) for S in (512, 1024, 2048, 4096, 8192, 16384, 32768)]
+    shapes += [("llama3 GQA 32/8 x 128", 4, 32, 8, 128, 4096, True), ("llama3 GQA 32/8 x 128", 1, 32, 8, 128, 4096, False)]
+    shapes += [("falcon MQA 71/1 x 64", 1, 71, 1, 64, S, True) for S in (1024, 2048, 4096, 8192, 16384)]
+    for label, B, Hq, Hkv, D, S, causal in shapes:
+        g = torch.Generator(device="cuda").manual_seed(42)
+        t = dict(Q=torch.randn(B, Hq, S, D, device="cuda", generator=g).half(),
+                 K=torch.randn(B, Hkv, S, D, device="cuda", generator=g).half(),
+                 V=torch.randn(B, Hkv, S, D, device="cuda", generator=g).half())
+        t["O"] = torch.zeros_like(t["Q"])
+        mod = m if causal else modules.get("vanilla", causal=False)
+        n = max(10, min(steps, int(2e13 / configs.attn_flops(B, Hq, S, S, D, causal))))
+        flops = configs.attn_flops(B, Hq, S, S, D, causal)
+        _, ev = graph_timed(mod, t, n, warmup, per_graph=min(20, n))
+        for x in "QKV":
+            t[x].zero_()
+        _, evz = graph_timed(mod, t, n, warmup, per_graph=min(20, n))
+        rows.append(dict(shape=label, batch=B, seq=S, causal=causal, us=round(ev * 1e3, 2), tflops=round(flops / ev / 1e9, 1),
+                         frac=round(flops / ev / 1e9 / configs.MFMA_F16_PEAK_TFLOPS, 4),
+                         zero_inputs_us=round(evz * 1e3, 2), zero_inputs_frac=round(flops / evz / 1e9 / configs.MFMA_F16_PEAK_TFLOPS, 4)))
+        del t
+        torch.cuda.empty_cache()
+    return rows
 
 
 def bench_rmsnorm(steps, warmup):
@@ -387,6 +418,8 @@ def main():
             torch.cuda.empty_cache()
     if wl == "decode" or (wl == "all" and not a.no_decode):
         extra["decode_append_M16_P1024"] = guarded(bench_decode, 100, a.warmup)
+    if wl == "sweep":
+        extra["attention_sweep"] = bench_sweep(a.steps, a.warmup)
     if van is None:                       # a single non-headline workload was asked for
         print(json.dumps({"workload": wl, **extra}))
         return
