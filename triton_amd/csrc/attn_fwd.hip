@@ -183,17 +183,21 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
                 }
             }
             fetch_noise(key0 + 64, gpre);    // the next block of the same parity, two pipeline steps ahead of its use
-            const float dmax = half_max(max16(d));             // (shared by the lane pair of a query, like m2)
-            const bool seen = dmax > -INFINITY;                // a block can be entirely masked for this row pair
-            const bool raise = dmax > 8.0f || (!have2 && seen);
-            if (__builtin_amdgcn_ballot_w64(raise) != 0) {     // wave-uniform; rare after a row's first block
+            // The test runs on the lane's own 16 keys; the exchange with the other lane of the query (m2 and have2 are
+            // shared by the pair) is made on the rare path only -- if either lane of a pair wants the raise, the
+            // wave-wide vote takes every lane there.
+            const float down = max16_bare(d);
+            if (__builtin_amdgcn_ballot_w64(down > 8.0f || (!have2 && down > -INFINITY)) != 0) {     // rare after a row's first block
+                const float dmax = half_max(down);
+                const bool seen = dmax > -INFINITY;            // a block can be entirely masked for this row pair
+                const bool raise = dmax > 8.0f || (!have2 && seen);
                 const float shift = raise ? dmax : 0.f;
                 l2 *= fast_exp2(-shift);
                 m2 += shift;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) d[r] -= shift;
+                have2 = have2 || seen;
             }
-            have2 = have2 || seen;
             float sum = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; ++r) sum += fast_exp2(d[r]);
@@ -207,10 +211,11 @@ __global__ __launch_bounds__(NW * 64, NW == 8 ? 1 : 2) void attn_fwd_kernel(cons
                 sx[r] = ok ? sx[r] : -INFINITY;      // (a select: stale-LDS garbage past the last block never propagates)
             }
         }
-        smax = half_max(max16(sx)) * a.c1;
+        smax = max16_bare(sx) * a.c1;          // over the lane's own keys; the pair's maximum is formed in rescale()
         return __builtin_amdgcn_ballot_w64(smax > m + 8.0f) != 0;
     };
-    auto rescale = [&](float smax) __attribute__((always_inline)) {
+    auto rescale = [&](float smax_own) __attribute__((always_inline)) {
+        const float smax = half_max(smax_own);
         const float mnew = fmaxf(m, smax);
         const float alpha = fast_exp2(m - mnew);
         l *= alpha;

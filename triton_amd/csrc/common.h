@@ -57,6 +57,25 @@ __device__ __forceinline__ float max16(const float16_t& s) {
     return fmaxf(max3(a, b, s[15]), max3(c, d, e));
 }
 
+// The same maximum issued as the bare instructions.  fmaxf on a value the compiler cannot prove to be no signalling
+// NaN (an MFMA result, a value that passed a select) is preceded by a canonicalising v_max_f32 x, x, x: 15 extra
+// instructions per 16 values.  The hardware maximum quiets NaNs by itself.  Only for values that were produced at least
+// one MFMA earlier: the compiler does not see which registers the instruction reads, so it inserts no wait states
+// between a matrix instruction and this read of its result.
+__device__ __forceinline__ float max3_bare(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
+__device__ __forceinline__ float max16_bare(const float16_t& s) {
+    const float a = max3_bare(s[0], s[1], s[2]), b = max3_bare(s[3], s[4], s[5]), c = max3_bare(s[6], s[7], s[8]);
+    const float d = max3_bare(s[9], s[10], s[11]), e = max3_bare(s[12], s[13], s[14]);
+    const float x = max3_bare(a, b, s[15]), y = max3_bare(c, d, e);
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 __device__ __forceinline__ float fast_rsqrt(float x) { return __builtin_amdgcn_rsqf(x); }
