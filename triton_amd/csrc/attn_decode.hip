@@ -45,6 +45,14 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * DV];
     __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * DV];
     __shared__ float st_m[DNW][32], st_l[DNW][32], st_m2[DNW][32], st_l2[DNW][32];
+    // K blocks are fetched as whole rows (a wave-wide load = 1 KB of consecutive bytes) and turned into MFMA operands
+    // through a wave-private LDS area: a load whose lanes each take 16 bytes of their own row -- the operand layout --
+    // is served at 16 bytes per clock (36 GB/s per CU measured), the row-wise one at 64 (130 GB/s).  Not with the whole
+    // head dimension of V in one workgroup at head_dim 128: the two V stages leave no room for the area.
+    constexpr bool KLDS = !(D == 128 && DS == 1);
+    constexpr int CPRK = D / 8;       // 16-byte chunks per K row
+    constexpr int RPIK = 64 / CPRK;   // K rows per wave-wide load
+    __shared__ __attribute__((aligned(1024))) half_t Kt[KLDS ? DNW * 32 * D : 8];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -75,12 +83,34 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     // ---- K: block rows straight into registers as A operands (lane: key c of the block, columns ks*16 + 8h ..)
     const __amdgpu_buffer_rsrc_t krs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(a.k + b * a.kb + kvh * a.kh), 0, (int)(((int64_t)(a.Skv - 1) * a.ks + D) * 2), 0x00020000);
-    const int kvo = (int)(c * a.ks * 2) + 16 * h;
-    const int kblk_bytes = (int)(32 * a.ks * 2);
+    const int kvo = KLDS ? (int)((lane / CPRK) * a.ks * 2) + (lane % CPRK) * 16 : (int)(c * a.ks * 2) + 16 * h;
+    const int kblk_bytes = (int)(32 * a.ks * 2), kpiece_bytes = (int)(RPIK * a.ks * 2);
+    // With KLDS the registers hold piece i = rows i*RPIK .. +RPIK-1 of the block as they lie in memory (D/16 = NS
+    // pieces); k_operands() below turns them into the operands in place.  Without it they are the operands.
     auto fetch_k = [&](int blk, half8_t (&ka)[NS]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int ks = 0; ks < NS; ++ks)
-            ka[ks] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvo + ks * 32, blk * kblk_bytes, 0));
+        for (int ks = 0; ks < NS; ++ks) {
+            if constexpr (KLDS)
+                ka[ks] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvo, blk * kblk_bytes + ks * kpiece_bytes, 0));
+            else
+                ka[ks] = __builtin_bit_cast(half8_t, __builtin_amdgcn_raw_buffer_load_b128(krs, kvo + ks * 32, blk * kblk_bytes, 0));
+        }
+    };
+    // Rows into the wave's area (chunk j of row r at j ^ swz<D>(r): the write of a piece covers its 1 KB once, and
+    // the 32 rows read back at one logical chunk touch every bank once), operands out of it.  LDS operations of one
+    // wave execute in order and nobody else touches the area: no barrier.
+    auto k_operands = [&](half8_t (&ka)[NS]) __attribute__((always_inline)) {
+        if constexpr (KLDS) {
+            half_t* kt = Kt + wave * 32 * D;
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                const int r = i * RPIK + lane / CPRK;
+                *reinterpret_cast<half8_t*>(&kt[r * D + (((lane % CPRK) ^ swz<D>(r)) << 3)]) = ka[i];
+            }
+#pragma unroll
+            for (int ks = 0; ks < NS; ++ks)
+                ka[ks] = *reinterpret_cast<const half8_t*>(&kt[c * D + (((2 * ks + h) ^ swz<D>(c)) << 3)]);
+        }
     };
     // ---- V: block rows global -> LDS, chunk c of row r stored at c ^ swz<D>(r); load n covers rows n*RPI + lane/CPR
     const __amdgpu_buffer_rsrc_t vrs = __builtin_amdgcn_make_buffer_rsrc(
@@ -157,6 +187,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         float16_t s;
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        k_operands(kc);
 #pragma unroll
         for (int ks = 0; ks < NS; ++ks) s = mfma32(kc[ks], qB[ks], s);
         if constexpr (NOISE) fetch_k(blk + DNW, kc);
@@ -436,6 +467,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             float16_t s;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s[r] = 0.f;
+            k_operands(kc);
 #pragma unroll
             for (int ks = 0; ks < NS; ++ks) s = mfma32(qB[ks], kc[ks], s);
             float x = 0.f, y = 0.f;
