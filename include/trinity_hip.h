@@ -114,7 +114,8 @@ int trn_attn_fwd_f16(const trn_attn_desc* desc, const void* q, const void* k, co
  * trn_attn_fwd_f16 with a caller-provided workspace.  In the reference every cross-kernel intermediate is a
  * caller-allocated tensor passed to `forward` (C, C_exp, C_sum ... in vanilla_llama_benchmark.py:42-77, zero-filled
  * by the driver, :237-240); this is that convention for the one intermediate these kernels have.  For decode shapes
- * (seq_q <= 32) with few heads the keys are then split over several workgroups per head, whose partial results and
+ * (seq_q <= 32) with fewer than 128 heads on a long cache (4096 keys or more with at most 16 heads, 8192 or more
+ * otherwise) the keys are then split over several workgroups per head, whose partial results and
  * arrival counters live in the workspace; for every other shape, or with workspace == NULL or too small, the call is
  * exactly trn_attn_fwd_f16.
  *   workspace        device memory, 256-byte aligned, trn_attn_workspace_bytes(desc) bytes, zero-filled ONCE before
@@ -192,8 +193,9 @@ int trn_attn_fwd_stats_f16(const trn_attn_desc* desc, const void* q, const void*
  * trn_attn_fwd_stats_f16 with a workspace, for few queries and few heads on a LONG cache: the reference's KeyFormer
  * and RoCo classes take any prefix length P (ref_rms.py:147-179, 249-280), and one workgroup per head sweeping tens
  * of thousands of keys leaves most of the chip idle.  trn_attn_stats_workspace_bytes(desc) says for which problems
- * the library would rather split (at most 32 queries per head, at most 48 heads in all, 8192 keys or more -- 4096
- * with at most 16 heads) and how many bytes that takes, 0 otherwise.  Given a zero-initialised workspace of at least
+ * the library would rather split (at most 32 queries per head, heads x head_dim at most 2048, and at least 8 keys per
+ * unit of that product -- 8192 keys for 8 heads of 128, 16384 for 16 -- but never fewer than 4096) and how many bytes
+ * that takes, 0 otherwise.  Given a zero-initialised workspace of at least
  * that many bytes (256-byte aligned, as for trn_attn_fwd_ws_f16) the attention runs with its keys split over
  * workgroups, and the statistics -- which need the merged row normalisers -- follow as a second launch over all keys
  * at once; lse (lse_pert with noise) is then required as the buffer that carries the normalisers between the two.

@@ -172,6 +172,26 @@ def test_no_workspace_exceeds_the_static_scratch_array(lib):
     assert 0 < largest <= capacity, (largest, capacity)
 
 
+def test_attention_split_rule_on_the_host(lib):
+    """trn_attn_workspace_bytes: keys are split from 4096 keys with at most 16 heads, from 8192 with more, never with 128
+    heads or more or with more than 32 queries per head; the size is counters + heads x shares x 32 x (head_dim + 4) floats."""
+    def need(heads, sq, skv, D=128, batch=1):
+        d = _desc(batch=batch, n_q_heads=heads, n_kv_heads=1, seq_q=sq, seq_kv=skv, head_dim=D, causal=0,
+                  q_stride_b=heads * sq * D, q_stride_h=sq * D, q_stride_s=D, k_stride_b=skv * D, k_stride_h=skv * D,
+                  k_stride_s=D, v_stride_b=skv * D, v_stride_h=skv * D, v_stride_s=D, o_stride_b=heads * sq * D,
+                  o_stride_h=sq * D, o_stride_s=D)
+        return lib.trn_attn_workspace_bytes(C.byref(d))
+    for heads, sq, skv, D, split in ((8, 16, 4096, 128, True), (8, 16, 4095, 128, False), (16, 1, 4096, 64, True),
+                                     (17, 16, 8191, 128, False), (17, 16, 8192, 128, True), (32, 16, 1040, 128, False),
+                                     (71, 16, 8192, 64, True), (127, 16, 8192, 128, True), (128, 16, 1 << 20, 128, False),
+                                     (8, 33, 16384, 128, False)):
+        assert (need(heads, sq, skv, D) > 0) == split, (heads, sq, skv, D)
+    assert need(64, 16, 4096, batch=2) == 0 and need(4, 16, 4096, batch=2) > 0      # the head count is batch x heads
+    # 32 heads, 8208 keys: 8 shares of 33 blocks; 8 heads, 4112 keys: 16 shares of 9 blocks, the last one short (15 shares)
+    assert need(32, 16, 8208) == 256 + 32 * 8 * 32 * 132 * 4
+    assert need(8, 16, 4112) == 256 + 8 * 15 * 32 * 132 * 4
+
+
 def test_statistics_split_rule_on_the_host(lib):
     """trn_attn_stats_workspace_bytes: the long-cache rule (few heads, many keys, at most 32 queries per head) is host
     arithmetic; where it says split, the size is that of the attention's own split workspace."""
@@ -181,9 +201,10 @@ def test_statistics_split_rule_on_the_host(lib):
                   k_stride_s=D, v_stride_b=skv * D, v_stride_h=skv * D, v_stride_s=D, o_stride_b=heads * sq * D,
                   o_stride_h=sq * D, o_stride_s=D)
         return fn(C.byref(d))
-    for heads, sq, skv, D, split in ((8, 16, 4096, 128, True), (8, 16, 4000, 128, False), (16, 16, 4096, 64, True),
-                                     (17, 16, 4096, 128, False), (32, 16, 8192, 128, True), (32, 16, 8191, 128, False),
-                                     (48, 4, 16384, 128, True), (49, 4, 16384, 128, False), (71, 16, 65536, 64, False),
+    for heads, sq, skv, D, split in ((8, 16, 8192, 128, True), (8, 16, 8191, 128, False), (16, 16, 8192, 64, True),
+                                     (16, 16, 8192, 128, False), (16, 16, 16384, 128, True), (4, 16, 4096, 128, True),
+                                     (4, 16, 4095, 128, False), (2, 16, 4096, 64, True), (17, 4, 65536, 128, False),
+                                     (32, 16, 65536, 128, False), (32, 16, 16384, 64, True), (71, 16, 65536, 64, False),
                                      (8, 33, 16384, 128, False), (8, 1, 1040, 128, False)):
         got = need(heads, sq, skv, D)
         assert (got > 0) == split, (heads, sq, skv, D, got)

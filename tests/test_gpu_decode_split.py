@@ -29,11 +29,11 @@ def workspace_for(q, k, v, o, scale, causal):
 
 SPLIT_CASES = [
     # B, Hq, Hkv, Sq, Skv, D, causal
-    (1, 32, 32, 16, 2064, 128, False),   # twice the reference's decode-append cache at Llama widths
-    (1, 32, 8, 16, 1552, 128, True),     # GQA, causal with a cached prefix
-    (1, 71, 1, 16, 3100, 64, False),     # Falcon: MQA, 71 heads of width 64
+    (1, 32, 32, 16, 8208, 128, False),   # eight times the reference's decode-append cache at Llama widths
+    (1, 32, 8, 16, 8200, 128, True),     # GQA, causal with a cached prefix
+    (1, 71, 1, 16, 8300, 64, False),     # Falcon: MQA, 71 heads of width 64
     (2, 4, 2, 1, 4099, 128, True),       # one query, ragged keys, many shares
-    (1, 3, 1, 32, 1569, 128, True),      # 50 blocks in shares of 7: the last share is short
+    (1, 3, 1, 32, 4129, 128, True),      # 130 blocks in shares of 9: the last share is short
     (1, 8, 8, 7, 20000, 128, False),     # long cache
 ]
 
@@ -64,7 +64,7 @@ def test_split_keys_match_oracle_and_unsplit(B, Hq, Hkv, Sq, Skv, D, causal):
 
 def test_split_keys_with_noise_and_fused_q_norm():
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D = 1, 8, 2, 16, 1552, 128
+    B, Hq, Hkv, Sq, Skv, D = 1, 8, 2, 16, 4112, 128
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=3)
     noise = ref.gumbel_noise((B, Hq, Sq, Skv), 99)
     tau, scale = 1.5, D ** -0.5
@@ -89,7 +89,7 @@ def test_split_keys_with_noise_and_fused_q_norm():
 
 def test_workspace_rules():
     from triton_amd import ops, _lib
-    q, k, v = make(1, 8, 8, 16, 1552, 128)
+    q, k, v = make(1, 8, 8, 16, 4112, 128)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     o = torch.zeros_like(qd)
     scale = 128 ** -0.5
@@ -105,8 +105,9 @@ def test_workspace_rules():
     with pytest.raises(_lib.TrnError) as e:
         ops.attention(qd, kd, vd, o, scale, False, workspace=big[16:16 + n])
     assert e.value.status_name == "TRN_E_ALIGN"
-    # shapes that do not split report 0 bytes: many heads, few keys, or more than 32 queries
-    for shape in ((1, 128, 128, 16, 1552, 128), (1, 8, 8, 16, 1040, 128), (1, 8, 8, 33, 1552, 128)):
+    # shapes that do not split report 0 bytes: many heads, too few keys for the head count, or more than 32 queries
+    for shape in ((1, 128, 1, 16, 8208, 128), (1, 8, 8, 16, 1040, 128), (1, 8, 8, 16, 4080, 128), (1, 32, 8, 16, 4112, 128),
+                  (1, 8, 8, 33, 4112, 128)):
         qq, kk, vv = (t.cuda() for t in make(*shape))
         assert ops.attention_workspace_bytes(qq, kk, vv, torch.zeros_like(qq), scale, False) == 0
     # a workspace handed to a shape that does not use one is ignored
@@ -120,7 +121,7 @@ def test_workspace_rules():
 def test_split_keys_under_graph_replay():
     """Captured once, replayed with eager work between the replays: every replay gives the eager result."""
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 1552, 128
+    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 8208, 128
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=17)
     scale = D ** -0.5
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
@@ -148,10 +149,10 @@ def test_split_keys_under_graph_replay():
 
 
 def test_decode_modules_split_path_matches_reference_classes():
-    """The decode-append modules at a shape where the attention splits its keys (8 heads, 1552 keys); RoCo asks for
+    """The decode-append modules at a shape where the attention splits its keys (8 heads, 4112 keys); RoCo asks for
     the key statistics, which are a second sweep of the one workgroup per head, so it is not split."""
     from triton_amd import modules
-    M, N, D, P = 16, 1024, 128, 1536
+    M, N, D, P = 16, 1024, 128, 4096
     H = N // D
     g = torch.Generator().manual_seed(5)
     cpu = dict(X=ref.reference_recipe((M, N), g) * 30, WQ=ref.reference_recipe((N, N), g) * 30,
@@ -181,8 +182,8 @@ def test_decode_modules_split_path_matches_reference_classes():
 # ---- trn_attn_fwd_stats_ws_f16: few heads on a long cache, keys split over workgroups, the statistics as a second launch
 STATS_SPLIT_CASES = [
     # B, Hq, Hkv, Sq, Skv, D, causal, with_noise
-    (1, 8, 8, 16, 4112, 128, True, False), (1, 8, 2, 16, 4112, 128, False, True), (1, 16, 4, 5, 8200, 64, True, True),
-    (1, 32, 8, 16, 8208, 128, True, False), (2, 3, 3, 32, 4099, 128, False, True), (1, 12, 12, 1, 9000, 64, True, False)]
+    (1, 8, 8, 16, 8208, 128, True, False), (1, 8, 2, 16, 8208, 128, False, True), (1, 16, 4, 5, 8200, 64, True, True),
+    (1, 32, 8, 16, 16400, 64, True, False), (2, 3, 3, 32, 6147, 128, False, True), (1, 12, 12, 1, 9000, 64, True, False)]
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,Sq,Skv,D,causal,with_noise", STATS_SPLIT_CASES)
@@ -230,18 +231,19 @@ def test_statistics_workspace_rule_and_fallbacks():
     for the row normalisers."""
     from triton_amd import ops
     scale = 0.125
-    for (B, Hq, Hkv, Sq, Skv, D), want_split in (((1, 71, 1, 16, 16400, 64), False), ((1, 32, 8, 16, 4112, 128), False),
-                                                  ((1, 8, 8, 16, 2064, 128), False), ((1, 8, 8, 33, 8208, 128), False),
-                                                  ((1, 32, 8, 16, 8208, 128), True), ((1, 16, 16, 4, 4112, 64), True)):
+    for (B, Hq, Hkv, Sq, Skv, D), want_split in (((1, 71, 1, 16, 16400, 64), False), ((1, 32, 8, 16, 16400, 128), False),
+                                                  ((1, 8, 8, 16, 4112, 128), False), ((1, 8, 8, 33, 8208, 128), False),
+                                                  ((1, 8, 8, 16, 8208, 128), True), ((1, 16, 16, 4, 8208, 64), True)):
         q = torch.zeros(B, Hq, Sq, D, dtype=torch.float16, device="cuda"); k = torch.zeros(B, Hkv, Skv, D, dtype=torch.float16, device="cuda")
         assert (ops.attention_stats_workspace_bytes(q, k, k, q, scale, True) > 0) == want_split, (Hq, Skv)
-    q, k, v = make(1, 8, 8, 16, 4112, 128, seed=29)
+    q, k, v = make(1, 8, 8, 16, 8208, 128, seed=29)
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
     n = ops.attention_stats_workspace_bytes(qd, kd, vd, qd, scale, True)
+    assert n > 0
     res = []
     for ws, with_lse in ((None, True), (torch.zeros(n // 2 // 256 * 256, dtype=torch.uint8, device="cuda"), True),
                          (torch.zeros(n, dtype=torch.uint8, device="cuda"), False)):
-        o = torch.zeros_like(qd); s1 = torch.zeros(1, 8, 4112, device="cuda"); lse = torch.zeros(1, 8, 16, device="cuda")
+        o = torch.zeros_like(qd); s1 = torch.zeros(1, 8, 8208, device="cuda"); lse = torch.zeros(1, 8, 16, device="cuda")
         ops.attention_with_stats(qd, kd, vd, o, scale, True, s1, None, lse=lse if with_lse else None, workspace=ws)
         torch.cuda.synchronize()
         res.append((o, s1))

@@ -198,10 +198,10 @@ def test_decode_append_modules_match_reference_classes(amp, M, N, D, P):
 
 @pytest.mark.parametrize("variant", ["keyformer", "roco"])
 def test_decode_score_modules_on_a_long_cache_split_their_keys(variant):
-    """Eight heads on a 4096-token cache: the modules take the library's split path (keys over workgroups, statistics as
+    """Eight heads on an 8192-token cache: the modules take the library's split path (keys over workgroups, statistics as
     a second launch) with the reference's fp16 tensors converted on the way; whole-module outputs against the oracle."""
     from triton_amd import modules, ops
-    M, N, D, P = 16, 1024, 128, 4096
+    M, N, D, P = 16, 1024, 128, 8192
     cpu, H = _decode_tensors(M, N, D, P, seed=9)
     W = (cpu["WQ"], cpu["WK"], cpu["WV"])
     t = {k: v.cuda() for k, v in cpu.items()}

@@ -110,7 +110,7 @@ def test_keyformer_any_key_count_padding_never_read(B, Hq, Hkv, Sq, Skv, D, caus
 
 def test_keyformer_split_keys_any_key_count():
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D, tau = 1, 8, 2, 16, 2067, 128, 1.5
+    B, Hq, Hkv, Sq, Skv, D, tau = 1, 8, 2, 16, 4115, 128, 1.5
     q, k, v = make(B, Hq, Hkv, Sq, Skv, D, seed=22)
     noise = ref.gumbel_noise((B, Hq, Sq, Skv), 78)
     scale = D ** -0.5

@@ -46,8 +46,8 @@ def _run_both(shape, causal, seed):
 def test_static_scratch_matches_caller_workspace_twice_second_smaller():
     from triton_amd import _lib
     assert _lib.load().trn_check_device() == 0
-    _run_both((1, 32, 8, 16, 4112, 128), True, seed=11)     # 32 heads x 8 shares
-    _run_both((1, 8, 2, 5, 1600, 128), False, seed=12)      # fewer heads, fewer keys, other share count
+    _run_both((1, 32, 8, 16, 8208, 128), True, seed=11)     # 32 heads x 8 shares
+    _run_both((1, 8, 2, 5, 4200, 128), False, seed=12)      # fewer heads, fewer keys, other share count
 
 
 def test_static_scratch_many_heads_two_shares_and_shapes_that_need_none():
@@ -74,7 +74,7 @@ def test_static_scratch_call_captured_into_a_graph_and_replayed():
     the array's address), replayed with the program's own eager work and synchronisations between the replays, every
     replay held to the eager result bit for bit -- on fresh inputs each time, so a replay that did nothing would show."""
     from triton_amd import ops
-    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 2064, 128
+    B, Hq, Hkv, Sq, Skv, D = 1, 32, 8, 16, 8208, 128
     q, k, v = _problem(B, Hq, Hkv, Sq, Skv, D, seed=21)
     scale = D ** -0.5
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()

@@ -507,15 +507,18 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #endif
 }
 
-// Keys are split over workgroups when one workgroup per head would leave most of the chip idle and a head has enough
-// key blocks to repay the merge: publishing, arriving and collecting cost 4 - 5 us, which is what some 40 blocks of a
-// 128-wide head (twice as many of a 64-wide one) take a single workgroup; the threshold is 48.  Measured with 16
-// queries per head, 32 heads of width 128: 1040 keys 14.8 -> 16 us (hence not split), 2064 keys 24 -> 21 us, 4112
-// keys 43 -> 25 us, 16400 keys 154 -> 51 us; 8 heads, 16400 keys 150 -> 27 us.  The caller provides the workspace
-// for the partial results.
+// Keys are split over workgroups when a head has enough of them to repay the merge (publishing, arriving and collecting
+// cost 4 - 5 us) and the split form's slower K path: with the head dimension of V in one workgroup there is no room for
+// the row-wise K fetch at head_dim 128, and the column shares of the unsplit form (up to four workgroups per head, each
+// with that fetch) already use half the chip at 32 heads.  Measured with 16 queries per head, unsplit / split, us:
+// 32 heads of 128: 2064 keys 13.9 / 22.2, 4112 keys 21.5 / 27.1, 8208 keys 36.7 / 34.8, 16400 keys 69 / 57, 65552 keys
+// 406 / 196; 8 heads of 128: 4112 keys 20.0 / 20.0, 8208 keys 35.0 / 22.6, 65552 keys 233 / 65; 4 heads: 4112 keys 19.7 /
+// 18.6; 71 heads of 64: 4112 keys 14.1 / 14.5, 8208 keys 23.9 / 18.9.  Hence: from 4096 keys with at most 16 heads, from
+// 8192 with more, never with 128 heads or more.  The caller provides the workspace for the partial results.
 static int decode_splits(int batch, int n_q_heads, int seq_kv, int head_dim) {
     const int n_bh = batch * n_q_heads, nblk = (seq_kv + 31) / 32;
-    if (n_bh >= 128 || (int64_t)nblk * head_dim < 48 * 128) return 1;
+    (void)head_dim;
+    if (n_bh >= 128 || seq_kv < (n_bh <= 16 ? 4096 : 8192)) return 1;
     const int ns = max(1, min(min(16, 256 / n_bh), nblk / 4));
     const int bps = (nblk + ns - 1) / ns;                 // blocks per share, as the kernel computes it
     return (nblk + bps - 1) / bps;                        // no empty share: the last one starts inside the keys

@@ -482,15 +482,17 @@ extern "C" int trn_attn_fwd_stats_f16(const trn_attn_desc* d, const void* q, con
 }
 
 // Where two launches (keys split over workgroups, then the statistics over all keys at once) beat the single launch
-// whose statistics sweep runs with one workgroup per head and column share.  Measured, 16 queries per head, microseconds
-// one launch / two launches: 8 heads of 128: 43 / 35 at 4 k keys, 156 / 52 at 16 k; 16 heads of 64: 30 / 30 at 4 k,
-// 55 / 41 at 8 k; 32 heads of 128: 45 / 52 at 4 k, 82 / 77 at 8 k, 169 / 130 at 16 k; 71 heads of 64: 33 / 60 at 4 k,
-// 126 / 182 at 16 k (that many heads fill the chip by themselves).
+// whose two sweeps run with one workgroup per head and column share.  Measured, 16 queries per head, microseconds one
+// launch / two launches, RoCo (KeyFormer): 8 heads of 128: 27 / 35 (33 / 30) at 4 k keys, 47 / 38 (59 / 39) at 8 k, 163 /
+// 78 (209 / 77) at 32 k; 16 heads of 64: 24 / 30 (33 / 31) at 4 k, 44 / 41 (60 / 42) at 8 k; 16 heads of 128: 48 / 55
+// (61 / 55) at 8 k, 87 / 81 (112 / 79) at 16 k; 32 heads of 128: 48 / 65 (59 / 64) at 8 k, 165 / 189 (207 / 183) at 32 k;
+// 48 heads: the single launch at every length.  The crossover follows the work per key, heads x head_dim: up to 2048 of
+// it, from 8 keys per unit (1024: 8192 keys, 2048: 16384), never below 4096 keys.
 extern "C" int64_t trn_attn_stats_workspace_bytes(const trn_attn_desc* d) {
     const int64_t need = trn_attn_workspace_bytes(d);
     if (need == 0) return 0;
-    const int64_t n_bh = (int64_t)d->batch * d->n_q_heads;
-    return n_bh <= 48 && d->seq_kv >= (n_bh <= 16 ? 4096 : 8192) ? need : 0;
+    const int64_t per_key = (int64_t)d->batch * d->n_q_heads * d->head_dim;
+    return per_key <= 2048 && d->seq_kv >= (8 * per_key > 4096 ? 8 * per_key : 4096) ? need : 0;
 }
 
 extern "C" int trn_attn_fwd_stats_ws_f16(const trn_attn_desc* d, const void* q, const void* k, const void* v, void* o,
