@@ -42,17 +42,19 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     constexpr int NI = 32 / RPI;  // such loads per 32-key V block
     // two V stages (each holds the eight waves' private parts), as two arrays: LDS reads are ordered after
     // outstanding global->LDS loads that may alias them, and only distinct variables are provably disjoint
+    // (With the whole head dimension of V in one workgroup at head_dim 128 a V stage is 64 KB: one stage then, refilled
+    // as soon as its block's P V is issued, so that the K area below still fits.)
+    constexpr bool VSINGLE = D == 128 && DS == 1;
     __shared__ __attribute__((aligned(1024))) half_t Vs0[DNW * 32 * DV];
-    __shared__ __attribute__((aligned(1024))) half_t Vs1[DNW * 32 * DV];
+    __shared__ __attribute__((aligned(1024))) half_t Vs1[VSINGLE ? 8 : DNW * 32 * DV];
     __shared__ float st_m[DNW][32], st_l[DNW][32], st_m2[DNW][32], st_l2[DNW][32];
     // K blocks are fetched as whole rows (a wave-wide load = 1 KB of consecutive bytes) and turned into MFMA operands
     // through a wave-private LDS area: a load whose lanes each take 16 bytes of their own row -- the operand layout --
-    // is served at 16 bytes per clock (36 GB/s per CU measured), the row-wise one at 64 (130 GB/s).  Not with the whole
-    // head dimension of V in one workgroup at head_dim 128: the two V stages leave no room for the area.
-    constexpr bool KLDS = !(D == 128 && DS == 1);
+    // is served at 16 bytes per clock (36 GB/s per CU measured), the row-wise one at 64 (130 GB/s).
+    constexpr bool KLDS = true;
     constexpr int CPRK = D / 8;       // 16-byte chunks per K row
     constexpr int RPIK = 64 / CPRK;   // K rows per wave-wide load
-    __shared__ __attribute__((aligned(1024))) half_t Kt[KLDS ? DNW * 32 * D : 8];
+    __shared__ __attribute__((aligned(1024))) half_t Kt[DNW * 32 * D];
 
     const int tid = threadIdx.x, lane = tid & 63, c = lane & 31, h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         const int blk = blk0 + wave + it * DNW, key0 = blk * 32;
         // (with noise the registers are short: K is then single-buffered, refilled as soon as the scores are issued)
         if constexpr (!NOISE) fetch_k(blk + DNW, kn);
-        TRN_FETCH_V(blk + DNW, Vn);
+        if constexpr (!VSINGLE) TRN_FETCH_V(blk + DNW, Vn);
         if constexpr (NOISE) fetch_noise(blk + DNW, gn);
         float16_t s;
 #pragma unroll
@@ -238,7 +240,8 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
         m = mnew;
         // this block's V has landed: behind it only the next block's NS + NI (+ 4 noise) requests were issued
-        constexpr int kBehind = NS + NI + (NOISE ? 4 : 0);
+        // (one V stage: its refill is issued behind the block's P V, so only K and noise requests are younger)
+        constexpr int kBehind = NS + (VSINGLE ? 0 : NI) + (NOISE ? 4 : 0);
         __builtin_amdgcn_s_waitcnt(0x0f70 | (kBehind & 15) | ((kBehind >> 4) << 14));
 #pragma unroll
         for (int i = 0; i < NSV; ++i) {
@@ -247,6 +250,14 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
             const half4_t hi = lds_read_tr16(vp + voff_hi[i % NDB]);
             const half8_t va = half8_t{lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
             oacc[i % NDB] = mfma32(va, pB[i / NDB], oacc[i % NDB]);
+        }
+        // (The refill must not overtake the stage's readers.  The compiler does not order the global->LDS load
+        // behind the transposing reads by itself -- left alone it moved the load in front of the last of them -- hence
+        // the scheduling fence; the wait makes the reads' return explicit.)
+        if constexpr (VSINGLE) {
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0)
+            TRN_FETCH_V(blk + DNW, Vn);
         }
     };
     fetch_k(blk0 + wave, ka0);
@@ -278,17 +289,18 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
     for (int ks = 0; ks < NS; ++ks) asm volatile("" ::"v"(qB[ks]));
     for (int it = 0; it < nmine; it += 2) {
         if constexpr (NOISE) {
-            block(it, ka0, ka0, Vs0, Vs1, g0, g1);
-            if (it + 1 < nmine) block(it + 1, ka0, ka0, Vs1, Vs0, g1, g0);
+            block(it, ka0, ka0, Vs0, VSINGLE ? Vs0 : Vs1, g0, g1);
+            if (it + 1 < nmine) block(it + 1, ka0, ka0, VSINGLE ? Vs0 : Vs1, Vs0, g1, g0);
         } else {
-            block(it, ka0, ka1, Vs0, Vs1, g0, g1);
-            if (it + 1 < nmine) block(it + 1, ka1, ka0, Vs1, Vs0, g1, g0);
+            block(it, ka0, ka1, Vs0, VSINGLE ? Vs0 : Vs1, g0, g1);
+            if (it + 1 < nmine) block(it + 1, ka1, ka0, VSINGLE ? Vs0 : Vs1, Vs0, g1, g0);
         }
     }
 #undef TRN_FETCH_V
 
     // ---- merge the eight waves' (m, l, O^T) through LDS.  Partial O^T as float4 quads [d/4][query]: the first half
     // of the columns in this wave's part of Vs0, the second half in its part of Vs1 (each exactly 32 * DV/2 floats).
+    half_t* const Vhi = VSINGLE ? Kt : Vs1;            // (one V stage: the K area, as large, takes the second half)
     l = half_sum(l);
     __builtin_amdgcn_s_waitcnt(0x0f70);                 // the look-ahead requests past the end have landed too
     if (h == 0) { st_m[wave][c] = m; st_l[wave][c] = l; }
@@ -301,7 +313,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int quad = db * 8 + 2 * r4 + h;             // columns 4 quad .. +3 of this workgroup's share
-            float4_t* part = reinterpret_cast<float4_t*>((quad < DV / 8 ? Vs0 : Vs1) + wave * 32 * DV);
+            float4_t* part = reinterpret_cast<float4_t*>((quad < DV / 8 ? Vs0 : Vhi) + wave * 32 * DV);
             part[(quad % (DV / 8)) * 32 + c] =
                 float4_t{oacc[db][r4 * 4], oacc[db][r4 * 4 + 1], oacc[db][r4 * 4 + 2], oacc[db][r4 * 4 + 3]};
         }
@@ -324,7 +336,7 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 #pragma unroll
         for (int qi = 0; qi < NQD; ++qi) {
             const int quad = min(dg + 16 * qi, DV / 4 - 1);   // d = 4*quad .. +3 (a group without a quad re-reads the last)
-            const half_t* base = quad < DV / 8 ? Vs0 : Vs1;
+            const half_t* base = quad < DV / 8 ? Vs0 : Vhi;
             const int ql = quad % (DV / 8);
             acc[qi] = float4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -508,13 +520,12 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
 }
 
 // Keys are split over workgroups when a head has enough of them to repay the merge (publishing, arriving and collecting
-// cost 4 - 5 us) and the split form's slower K path: with the head dimension of V in one workgroup there is no room for
-// the row-wise K fetch at head_dim 128, and the column shares of the unsplit form (up to four workgroups per head, each
-// with that fetch) already use half the chip at 32 heads.  Measured with 16 queries per head, unsplit / split, us:
-// 32 heads of 128: 2064 keys 13.9 / 22.2, 4112 keys 21.5 / 27.1, 8208 keys 36.7 / 34.8, 16400 keys 69 / 57, 65552 keys
-// 406 / 196; 8 heads of 128: 4112 keys 20.0 / 20.0, 8208 keys 35.0 / 22.6, 65552 keys 233 / 65; 4 heads: 4112 keys 19.7 /
-// 18.6; 71 heads of 64: 4112 keys 14.1 / 14.5, 8208 keys 23.9 / 18.9.  Hence: from 4096 keys with at most 16 heads, from
-// 8192 with more, never with 128 heads or more.  The caller provides the workspace for the partial results.
+// cost 4 - 5 us) against the unsplit form, whose column shares (up to four workgroups per head) already use half the chip
+// at 32 heads.  Measured with 16 queries per head, unsplit / split, us: 32 heads of 128: 2064 keys 13.9 / 22.2, 4112 keys
+// 21.5 / 27.1, 8208 keys 36.7 / 35.8, 16400 keys 69 / 57, 65552 keys 406 / 198; 8 heads of 128: 4112 keys 20.0 / 18.1, 8208
+// keys 35 / 22, 65552 keys 232 / 59; 71 heads of 64: 4112 keys 14.1 / 14.5, 8208 keys 23.9 / 18.9.  Hence: from 4096 keys
+// with at most 16 heads, from 8192 with more, never with 128 heads or more.  The caller provides the workspace for the
+// partial results.
 static int decode_splits(int batch, int n_q_heads, int seq_kv, int head_dim) {
     const int n_bh = batch * n_q_heads, nblk = (seq_kv + 31) / 32;
     (void)head_dim;
