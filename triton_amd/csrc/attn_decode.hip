@@ -184,7 +184,13 @@ __global__ __launch_bounds__(DNW * 64, 1) void attn_decode_kernel(const AttnArgs
         const int blk = blk0 + wave + it * DNW, key0 = blk * 32;
         // (with noise the registers are short: K is then single-buffered, refilled as soon as the scores are issued)
         if constexpr (!NOISE) fetch_k(blk + DNW, kn);
-        if constexpr (!VSINGLE) TRN_FETCH_V(blk + DNW, Vn);
+        if constexpr (!VSINGLE) {
+            // (Vn is the stage the previous block read: the same fence as for the single stage below, so that the order
+            // does not hang on where the compiler happens to cut its scheduling regions)
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0)
+            TRN_FETCH_V(blk + DNW, Vn);
+        }
         if constexpr (NOISE) fetch_noise(blk + DNW, gn);
         float16_t s;
 #pragma unroll
