@@ -47,6 +47,12 @@ CASES = [
     (1, 4, 2, 32, 32, 128, True),
     (3, 4, 4, 32, 5000, 128, False),
     (1, 4, 2, 33, 1040, 128, True),      # one query more: back to the prefill kernel
+    # head_dim 128 with one workgroup per head (a single V stage, refilled behind its last reader): too few keys for
+    # column shares, and too many heads for them; several blocks per wave, causal and not
+    (1, 8, 8, 16, 216, 128, True),
+    (1, 8, 2, 16, 64, 128, False),
+    (1, 136, 8, 16, 1040, 128, True),
+    (2, 80, 80, 5, 2100, 128, False),
     (1, 64, 8, 1990, 2100, 128, True),   # 8-wave workgroups under a causal mask with a cached prefix and ragged ends:
                                          # the waves of a workgroup stop at different tiles
     (1, 16, 16, 520, 520, 64, True),     # head_dim 64 stays on 4-wave workgroups; a last workgroup of 8 queries
